@@ -35,6 +35,8 @@ class Architecture:
     # named raw configurations of this architecture (config.json keys) that a model name may
     # stand for instead of a folder: small random models for trying the engine out
     presets: tuple = ()      # ((name, raw config dict), ...)
+    # (config, name -> stored shape) -> config: sizes that only the checkpoint's tensors give
+    complete_config: Callable[[Any, Callable], Any] = None
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}
@@ -49,7 +51,7 @@ def register_architecture(entry: Architecture) -> Architecture:
 
 def _load_builtin():
     # Importing the module registers it.
-    from ..model import gpt2  # noqa: F401
+    from ..model import gpt2, kosesun  # noqa: F401
 
 
 def find_preset(name: str):
@@ -71,6 +73,8 @@ def resolve_architecture(raw_config: dict) -> Architecture:
     """The entry for a ``config.json`` dict, or one clear error listing what exists."""
     _load_builtin()
     names = raw_config.get("architectures")
+    if names is None and isinstance(raw_config.get("architecture"), str):
+        names = [raw_config["architecture"]]     # the key as a single name
     if isinstance(names, (list, tuple)) and names:
         name = names[0]
         if name in ARCHITECTURES:

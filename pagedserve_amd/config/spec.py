@@ -106,6 +106,10 @@ class ModelSpec:
     # how token ids become rows of the stream, and how the last rows become logits
     embedding: PartSpec = PartSpec("lookup")
     head: PartSpec = PartSpec("linear")
+    # 0: one residual stream of the width.  n >= 1: the stream is kept in n copies (rows of
+    # n * width floats): all equal to the embedding at the start, summed before the final norm;
+    # the blocks' arrangements say how a sublayer reads and writes them.
+    streams: int = 0
 
     def __post_init__(self):
         if not self.blocks:

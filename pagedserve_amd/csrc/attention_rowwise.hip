@@ -8,6 +8,7 @@
 // accumulators are float whatever the storage type.  Used for every token in the 32-bit path
 // and as the fallback for shapes the tiled kernels refuse; it reads keys that the step has
 // already stored, so prompt portions, whole prompts and decoded tokens are the same case.
+// `sink` (one float per head, or null) adds exp(sink[head]) to the softmax's denominator.
 #include <math.h>
 
 #include "common.h"
@@ -21,7 +22,8 @@ __global__ __launch_bounds__(64) void attention_rowwise_kernel(
     const T* __restrict__ v_pool, T* __restrict__ out, int64_t out_stride,
     const int* __restrict__ tok_list, const int* __restrict__ tok_item,
     const int* __restrict__ tok_pos, const int* __restrict__ tables, int table_width, int heads,
-    int kv_heads, int head_dim, int page_size, int num_pages, float scale, int window) {
+    int kv_heads, int head_dim, int page_size, int num_pages, float scale, int window,
+    const float* __restrict__ sink) {
   __shared__ float q_row[256];
   __shared__ float prob[64];
   __shared__ int64_t key_base[64];
@@ -39,8 +41,9 @@ __global__ __launch_bounds__(64) void attention_rowwise_kernel(
     q_row[i] = to_float<T>(q[(int64_t)t * q_stride + (int64_t)head * head_dim + i]);
   __syncthreads();
 
-  float running_max = -INFINITY;
-  float running_sum = 0.f;
+  // a sink is a score without a key or a value: it only takes part in the denominator
+  float running_max = sink ? sink[head] : -INFINITY;
+  float running_sum = sink ? 1.f : 0.f;
   float acc[AR_MAX_DIMS] = {0.f, 0.f, 0.f, 0.f};
 
   for (int k0 = first_key; k0 < end_key; k0 += 64) {
@@ -100,7 +103,7 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
                                     const int* tables, int table_width, int tokens, int heads,
                                     int kv_heads,
                                     int head_dim, int page_size, int num_pages, float scale,
-                                    int window, int dtype, void* stream) {
+                                    int window, const float* sink, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_rowwise: bad sizes");
@@ -118,12 +121,12 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
     hipLaunchKernelGGL(attention_rowwise_kernel<float>, grid, dim3(64), 0, s, (const float*)q,
                        q_stride, (const float*)k_pool, (const float*)v_pool, (float*)out,
                        out_stride, tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads,
-                       head_dim, page_size, num_pages, scale, window);
+                       head_dim, page_size, num_pages, scale, window, sink);
   else
     hipLaunchKernelGGL(attention_rowwise_kernel<bf16_t>, grid, dim3(64), 0, s, (const bf16_t*)q,
                        q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out,
                        out_stride, tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads,
-                       head_dim, page_size, num_pages, scale, window);
+                       head_dim, page_size, num_pages, scale, window, sink);
   PS_CHECK_LAUNCH("ps_attention_rowwise");
   return 0;
 }

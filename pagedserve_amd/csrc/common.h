@@ -16,6 +16,7 @@ enum PsEpilogue {
   PS_EPI_GELU_TANH = 1,  // C = gelu_tanh(A W^T + b)
   PS_EPI_GELU_ERF = 2,   // C = gelu_erf(A W^T + b)
   PS_EPI_RESIDUAL = 3,   // C(float) += A W^T + b   (C holds the residual stream)
+  PS_EPI_RELU2 = 4,      // C = max(A W^T + b, 0)^2
 };
 
 struct bf16_t {
@@ -202,6 +203,10 @@ template <int EPI>
 __device__ inline float apply_activation(float v) {
   if (EPI == PS_EPI_GELU_TANH) return gelu_tanh_f(v);
   if (EPI == PS_EPI_GELU_ERF) return gelu_erf_f(v);
+  if (EPI == PS_EPI_RELU2) {
+    const float r = fmaxf(v, 0.f);
+    return r * r;
+  }
   return v;
 }
 

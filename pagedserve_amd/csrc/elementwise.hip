@@ -343,3 +343,18 @@ extern "C" int ps_kv_write(const void* k, const void* v, int64_t stride, void* k
   PS_CHECK_LAUNCH("ps_kv_write");
   return 0;
 }
+
+// logits <- cap * tanh(logits / cap)
+__global__ void softcap_kernel(float* __restrict__ logits, int64_t ld, int vocab, float cap) {
+  float* row = logits + (int64_t)blockIdx.x * ld;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) row[i] = cap * tanhf(row[i] / cap);
+}
+
+extern "C" int ps_softcap(float* logits, int64_t ld, int rows, int vocab, float cap, void* stream) {
+  PS_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab && cap > 0.f, "ps_softcap: bad sizes");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(softcap_kernel, dim3(rows), dim3(vocab >= 1024 ? 1024 : 256), 0,
+                     (hipStream_t)stream, logits, ld, vocab, cap);
+  PS_CHECK_LAUNCH("ps_softcap");
+  return 0;
+}

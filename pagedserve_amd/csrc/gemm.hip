@@ -36,7 +36,7 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
              p->c_dtype);
   PS_REQUIRE(!(p->dtype == PS_F32 && p->c_dtype == PS_BF16),
              "ps_linear: float operands with bfloat16 output are not supported");
-  PS_REQUIRE(p->epilogue >= PS_EPI_NONE && p->epilogue <= PS_EPI_RESIDUAL,
+  PS_REQUIRE(p->epilogue >= PS_EPI_NONE && p->epilogue <= PS_EPI_RELU2,
              "ps_linear: unknown epilogue %d", p->epilogue);
   PS_REQUIRE(p->epilogue != PS_EPI_RESIDUAL || p->c_dtype == PS_F32,
              "ps_linear: the residual epilogue needs a float output");

@@ -469,6 +469,7 @@ static int launch_tiled(const void* a, const void* w, const float* bias, void* c
     case PS_EPI_NONE: PS_LAUNCH_TG(PS_EPI_NONE); break;
     case PS_EPI_GELU_TANH: PS_LAUNCH_TG(PS_EPI_GELU_TANH); break;
     case PS_EPI_GELU_ERF: PS_LAUNCH_TG(PS_EPI_GELU_ERF); break;
+    case PS_EPI_RELU2: PS_LAUNCH_TG(PS_EPI_RELU2); break;
     case PS_EPI_RESIDUAL: PS_LAUNCH_TG(PS_EPI_RESIDUAL); break;
     default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
   }
@@ -588,6 +589,7 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
     PS_SKINNY_CASE(PS_EPI_NONE);
     PS_SKINNY_CASE(PS_EPI_GELU_TANH);
     PS_SKINNY_CASE(PS_EPI_GELU_ERF);
+    PS_SKINNY_CASE(PS_EPI_RELU2);
     PS_SKINNY_CASE(PS_EPI_RESIDUAL);
     default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
   }

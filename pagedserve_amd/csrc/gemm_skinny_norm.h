@@ -250,6 +250,7 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
     PS_NORM_CASE(PS_EPI_NONE);
     PS_NORM_CASE(PS_EPI_GELU_TANH);
     PS_NORM_CASE(PS_EPI_GELU_ERF);
+    PS_NORM_CASE(PS_EPI_RELU2);
     PS_NORM_CASE(PS_EPI_RESIDUAL);
     default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
   }

@@ -267,6 +267,7 @@ static int launch_wide(const void* a, const void* wp, const float* bias, void* c
     case PS_EPI_NONE: PS_LAUNCH_GW(PS_EPI_NONE); break;
     case PS_EPI_GELU_TANH: PS_LAUNCH_GW(PS_EPI_GELU_TANH); break;
     case PS_EPI_GELU_ERF: PS_LAUNCH_GW(PS_EPI_GELU_ERF); break;
+    case PS_EPI_RELU2: PS_LAUNCH_GW(PS_EPI_RELU2); break;
     case PS_EPI_RESIDUAL: PS_LAUNCH_GW(PS_EPI_RESIDUAL); break;
     default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
   }

@@ -1,0 +1,189 @@
+// Gated linear attention: a recurrent mixer whose state is a matrix per head.
+//
+//   S_t = diag(alpha_t) S_(t-1) + k_t v_t^T        (S: [key_dim, value_dim], float, per request)
+//   o_t = S_t^T q_t
+//
+// with a decay alpha in (0, 1) per key channel, alpha = sigmoid(z)^(1/tau), z a low-rank
+// projection of the layer's input.  Three launches: the decays of the step's tokens, the
+// recurrence, and the output's norm and gate.  The state, the decays and everything they are
+// made from are 32-bit; q, k, v arrive as the float columns of the layer's projection.
+#include <math.h>
+
+#include "common.h"
+#include "pagedserve_hip.h"
+
+// alpha[t, c] = exp(log_sigmoid(z) / tau), z = bias[c] + sum_r low[t, r] w[c, r].
+template <typename T>
+__global__ __launch_bounds__(256) void gla_decay_kernel(
+    const float* __restrict__ proj, int64_t ld, int low_col, int rank, const T* __restrict__ w,
+    const float* __restrict__ bias, float inv_tau, float* __restrict__ alpha, int channels) {
+  extern __shared__ float low[];
+  const int t = blockIdx.x;
+  for (int r = threadIdx.x; r < rank; r += blockDim.x) low[r] = proj[(int64_t)t * ld + low_col + r];
+  __syncthreads();
+  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    float z = bias ? bias[c] : 0.f;
+    const T* w_row = w + (int64_t)c * rank;
+    for (int r = 0; r < rank; ++r) z = fmaf(low[r], to_float<T>(w_row[r]), z);
+    // log sigmoid(z) = min(z, 0) - log(1 + exp(-|z|))
+    const float log_sigmoid = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+    alpha[(int64_t)t * channels + c] = expf(log_sigmoid * inv_tau);
+  }
+}
+
+#define GLA_COLS 16    // value columns per block (one wave): lane = row group * 16 + column
+#define GLA_CHUNK 8    // tokens whose q, k, alpha are staged in LDS at a time
+
+// A block owns GLA_COLS columns of one head's state for one item of the step and walks the
+// item's tokens in order.  The state's rows are dealt to four row groups, RPL rows per lane,
+// in registers; o needs the sum over the row groups (two lane exchanges per token).
+template <int RPL>
+__global__ __launch_bounds__(64) void gla_scan_kernel(
+    const float* __restrict__ proj, int64_t ld, int q_col, int k_col, int v_col,
+    const float* __restrict__ alpha, float* __restrict__ state, float* __restrict__ out,
+    const int* __restrict__ cu_tokens, const int* __restrict__ slots, int heads, int key_dim,
+    int value_dim, float q_scale) {
+  constexpr int PAD = RPL + 4;   // row groups start in different banks
+  __shared__ float s_q[GLA_CHUNK][4 * PAD];
+  __shared__ float s_k[GLA_CHUNK][4 * PAD];
+  __shared__ float s_a[GLA_CHUNK][4 * PAD];
+  __shared__ float s_v[GLA_CHUNK][GLA_COLS];
+  const int item = blockIdx.x, head = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int col = blockIdx.z * GLA_COLS + (lane & 15);
+  const int group = lane >> 4;
+  const bool has_col = col < value_dim;
+  const int t0 = cu_tokens[item], t1 = cu_tokens[item + 1];
+  const int slot = slots[item];
+  float* s_ptr = state + (((int64_t)slot * heads + head) * key_dim) * value_dim;
+  float S[RPL];
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int r = group * RPL + i;
+    S[i] = (r < key_dim && has_col) ? s_ptr[(int64_t)r * value_dim + col] : 0.f;
+  }
+  const int channels = heads * key_dim;
+  for (int base = t0; base < t1; base += GLA_CHUNK) {
+    const int count = (t1 - base) < GLA_CHUNK ? (t1 - base) : GLA_CHUNK;
+    __syncthreads();
+    for (int idx = lane; idx < GLA_CHUNK * 4 * RPL; idx += 64) {
+      const int tt = idx / (4 * RPL);
+      const int r = idx - tt * (4 * RPL);
+      const bool valid = tt < count && r < key_dim;
+      const int64_t t = base + (tt < count ? tt : 0);
+      const int c = head * key_dim + (r < key_dim ? r : 0);
+      const float qv = proj[t * ld + q_col + c], kv = proj[t * ld + k_col + c];
+      const float av = alpha[t * channels + c];
+      const int at = (r / RPL) * PAD + (r % RPL);
+      s_q[tt][at] = valid ? qv * q_scale : 0.f;
+      s_k[tt][at] = valid ? kv : 0.f;
+      s_a[tt][at] = valid ? av : 0.f;
+    }
+    for (int idx = lane; idx < GLA_CHUNK * GLA_COLS; idx += 64) {
+      const int tt = idx / GLA_COLS;
+      const int c = blockIdx.z * GLA_COLS + (idx - tt * GLA_COLS);
+      const bool valid = tt < count && c < value_dim;
+      const int64_t t = base + (tt < count ? tt : 0);
+      const float vv = proj[t * ld + v_col + head * value_dim + (c < value_dim ? c : 0)];
+      s_v[tt][idx - tt * GLA_COLS] = valid ? vv : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < count; ++tt) {
+      const float v = s_v[tt][lane & 15];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < RPL; ++i) {
+        const int at = group * PAD + i;
+        S[i] = fmaf(s_a[tt][at], S[i], s_k[tt][at] * v);
+        o = fmaf(S[i], s_q[tt][at], o);
+      }
+      o = xor_sum<16>(o);
+      o = xor_sum<32>(o);
+      if (group == 0 && has_col)
+        out[(int64_t)(base + tt) * heads * value_dim + head * value_dim + col] = o;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int r = group * RPL + i;
+    if (r < key_dim && has_col) s_ptr[(int64_t)r * value_dim + col] = S[i];
+  }
+}
+
+// out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w * silu(gate[t, h, :]).
+template <typename T>
+__global__ __launch_bounds__(64) void gla_output_kernel(
+    const float* __restrict__ o, const float* __restrict__ w, float eps,
+    const float* __restrict__ gate, int64_t gate_ld, T* __restrict__ out, int64_t out_stride,
+    int heads, int value_dim) {
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const float* row = o + ((int64_t)t * heads + head) * value_dim;
+  float sum = 0.f;
+  for (int d = lane; d < value_dim; d += 64) sum = fmaf(row[d], row[d], sum);
+  const float inv = 1.0f / sqrtf(wave_sum(sum) / (float)value_dim + eps);
+  for (int d = lane; d < value_dim; d += 64) {
+    const float g = gate[(int64_t)t * gate_ld + head * value_dim + d];
+    const float silu = g / (1.0f + expf(-g));
+    out[(int64_t)t * out_stride + head * value_dim + d] = from_float<T>(row[d] * inv * w[d] * silu);
+  }
+}
+
+extern "C" int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank, const void* w,
+                            const float* bias, float tau, float* alpha, int tokens, int channels,
+                            int dtype, void* stream) {
+  PS_REQUIRE(tokens >= 0 && rank > 0 && channels > 0 && tau > 0.f, "ps_gla_decay: bad sizes");
+  PS_REQUIRE(rank <= 8192, "ps_gla_decay: rank %d above 8192", rank);
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_gla_decay: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t lds = (size_t)rank * sizeof(float);
+  if (dtype == PS_F32)
+    hipLaunchKernelGGL(gla_decay_kernel<float>, dim3(tokens), dim3(256), lds, s, proj, ld, low_col,
+                       rank, (const float*)w, bias, 1.0f / tau, alpha, channels);
+  else
+    hipLaunchKernelGGL(gla_decay_kernel<bf16_t>, dim3(tokens), dim3(256), lds, s, proj, ld, low_col,
+                       rank, (const bf16_t*)w, bias, 1.0f / tau, alpha, channels);
+  PS_CHECK_LAUNCH("ps_gla_decay");
+  return 0;
+}
+
+extern "C" int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
+                           const float* alpha, float* state, float* out, const int* cu_tokens,
+                           const int* slots, int items, int max_slots, int heads, int key_dim,
+                           int value_dim, float q_scale, void* stream) {
+  PS_REQUIRE(items >= 0 && heads > 0 && key_dim > 0 && value_dim > 0 && max_slots > 0,
+             "ps_gla_scan: bad sizes");
+  PS_REQUIRE(key_dim <= 256, "ps_gla_scan: key head size %d above 256", key_dim);
+  PS_REQUIRE(heads <= 65535 && (value_dim + GLA_COLS - 1) / GLA_COLS <= 65535, "ps_gla_scan: grid too large");
+  if (items == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(items, heads, (value_dim + GLA_COLS - 1) / GLA_COLS);
+#define PS_LAUNCH_GLA(RPL)                                                                       \
+  hipLaunchKernelGGL((gla_scan_kernel<RPL>), grid, dim3(64), 0, s, proj, ld, q_col, k_col, v_col, \
+                     alpha, state, out, cu_tokens, slots, heads, key_dim, value_dim, q_scale)
+  if (key_dim <= 32) PS_LAUNCH_GLA(8);
+  else if (key_dim <= 64) PS_LAUNCH_GLA(16);
+  else if (key_dim <= 128) PS_LAUNCH_GLA(32);
+  else PS_LAUNCH_GLA(64);
+#undef PS_LAUNCH_GLA
+  PS_CHECK_LAUNCH("ps_gla_scan");
+  return 0;
+}
+
+extern "C" int ps_gla_output(const float* o, const float* w, float eps, const float* gate,
+                             int64_t gate_ld, void* out, int64_t out_stride, int tokens, int heads,
+                             int value_dim, int dtype, void* stream) {
+  PS_REQUIRE(tokens >= 0 && heads > 0 && value_dim > 0 && eps > 0.f && heads <= 65535,
+             "ps_gla_output: bad sizes");
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_gla_output: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    hipLaunchKernelGGL(gla_output_kernel<float>, dim3(tokens, heads), dim3(64), 0, s, o, w, eps, gate,
+                       gate_ld, (float*)out, out_stride, heads, value_dim);
+  else
+    hipLaunchKernelGGL(gla_output_kernel<bf16_t>, dim3(tokens, heads), dim3(64), 0, s, o, w, eps, gate,
+                       gate_ld, (bf16_t*)out, out_stride, heads, value_dim);
+  PS_CHECK_LAUNCH("ps_gla_output");
+  return 0;
+}

@@ -114,11 +114,13 @@ int ps_kv_write(const void* k, const void* v, int64_t stride, void* k_pool, void
 // Attention of `tokens` tokens of the step (those listed in tok_list, or all when it is
 // null) over their requests' cached keys 0..position (or the last `window` of them), one
 // wave per (token, head).  Any head_dim from 1 to 256; heads must be a multiple of kv_heads.
+// sink: null, or one float per head that enters the softmax's denominator as exp(sink[head])
+// (a score without key or value, not scaled); the same in the attention kernels below.
 int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                          void* out, int64_t out_stride, const int* tok_list, const int* tok_item,
                          const int* tok_pos, const int* tables, int table_width, int tokens,
                          int heads, int kv_heads, int head_dim, int page_size, int num_pages,
-                         float scale, int window, int dtype, void* stream);
+                         float scale, int window, const float* sink, int dtype, void* stream);
 
 // The same result in true 32-bit for the items of several tokens (prompt portions), a block
 // of four waves per (tile of ps_attention_tiled_f32_tile() queries, head): float pools, float
@@ -237,6 +239,60 @@ int ps_graph_end(void* stream, void** exec_out, int* node_count);
 int ps_graph_abort(void* stream);
 int ps_graph_launch(void* exec, void* stream);
 int ps_graph_destroy(void* exec);
+
+// ---- several copies of the residual stream -----------------------------------------------
+// x: [tokens, streams, width] float.  One launch does, per token:
+//   * if y != null:       x'_t = sum_s mix[s * streams + t] x_s + out_w[t] * y   (all t at once)
+//   * if normed != null:  u = sum_s in_w[s] x'_s;  normed = u / sqrt(mean(u^2) + eps) * gamma
+//   * if zero != null:    zero[token, :] = 0        (may be the buffer that y was read from)
+int ps_hyper_step(float* x, const float* y, const float* mix, const float* out_w,
+                  const float* in_w, const float* gamma, float eps, void* normed, float* zero,
+                  int tokens, int width, int streams, int out_dtype, void* stream);
+// x[t, s, :] = e[t, :];   out[r, :] = sum_s x[rows ? rows[r] : r, s, :].
+int ps_streams_expand(const float* e, float* x, int tokens, int width, int streams, void* stream);
+int ps_streams_collapse(const float* x, const int* rows, float* out, int n_rows, int width,
+                        int streams, void* stream);
+
+// ---- attention: what lies between the projection and the attention kernels ---------------
+// proj: [tokens, ld] float with the query, key and value columns at q_col, k_col, v_col
+// (heads * key_dim, kv_heads * key_dim, kv_heads * value_dim of them).  Queries and keys are
+// normed over their whole row (q_gamma / k_gamma: a weight per column, null: no norm), rotated
+// on the first rot_dims dimensions of every head (dimension 2i with 2i+1, angle position *
+// freqs[i]), values are kept (v_mode 1: v_first[t] = v) or mixed (v_mode 2: v = (1 - *v_lambda)
+// v + *v_lambda v_first[t]); keys and values go into their pages, queries to q_out, every head
+// cache_dim wide with zeros behind its own size.
+int ps_attention_prepare(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
+                         void* q_out, int64_t q_stride, void* k_pool, void* v_pool,
+                         const float* q_gamma, const float* k_gamma, float eps, const float* freqs,
+                         int rot_dims, void* v_first, const float* v_lambda, int v_mode,
+                         const int* tok_item, const int* tok_pos, const int* tables,
+                         int table_width, int tokens, int heads, int kv_heads, int key_dim,
+                         int value_dim, int cache_dim, int page_size, int num_pages, int dtype,
+                         void* stream);
+// ctx[t, h, :] *= sigmoid(gate[t * gate_ld + h]).
+int ps_head_gate(void* ctx, int64_t stride, const float* gate, int64_t gate_ld, int tokens,
+                 int heads, int head_dim, int dtype, void* stream);
+
+// ---- gated linear attention ----------------------------------------------------------------
+// alpha[t, c] = sigmoid(z)^(1 / tau) with z = bias[c] + sum_r proj[t, low_col + r] w[c, r].
+int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank, const void* w,
+                 const float* bias, float tau, float* alpha, int tokens, int channels, int dtype,
+                 void* stream);
+// For every item i of the step (tokens cu_tokens[i] .. cu_tokens[i + 1] - 1, state slot
+// slots[i]) and head: S = diag(alpha_t) S + k_t v_t^T, out[t] = S^T (q_t * q_scale), token after
+// token; state: [max_slots, heads, key_dim, value_dim] float, read at the start and written
+// back at the end; out: [tokens, heads * value_dim] float.
+int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
+                const float* alpha, float* state, float* out, const int* cu_tokens,
+                const int* slots, int items, int max_slots, int heads, int key_dim, int value_dim,
+                float q_scale, void* stream);
+// out[t, h, :] = rms_norm(o[t, h, :]) * w * silu(gate[t * gate_ld + h * value_dim ...]).
+int ps_gla_output(const float* o, const float* w, float eps, const float* gate, int64_t gate_ld,
+                  void* out, int64_t out_stride, int tokens, int heads, int value_dim, int dtype,
+                  void* stream);
+
+// logits[r, :vocab] = cap * tanh(logits[r, :vocab] / cap), rows ld floats apart.
+int ps_softcap(float* logits, int64_t ld, int rows, int vocab, float cap, void* stream);
 
 #ifdef __cplusplus
 }

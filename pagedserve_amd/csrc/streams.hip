@@ -1,0 +1,163 @@
+// Several copies of the residual stream ("hyper-connections"): X is [tokens, streams, width]
+// in float.  A sublayer reads a weighted sum of the copies and writes its result y back into
+// every copy while the copies are mixed with each other:
+//
+//   read:   u = sum_s in[s] X_s,  normed = u / sqrt(mean(u^2) + eps) * gamma
+//   write:  X'_t = sum_s mix[s, t] X_s + out[t] y          (all t from the old copies)
+//
+// One kernel does a write, a read, or a write followed by the read of the next sublayer
+// (the copies then make one trip through memory for both), and clears the buffer that the
+// next sublayer's products add their result into.  Everything is 32-bit.
+#include <math.h>
+
+#include "common.h"
+#include "pagedserve_hip.h"
+
+#define HS_MAX_STREAMS 8
+#define HS_THREADS 256
+
+template <typename TOut, int PER>
+__global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
+    float* __restrict__ X, const float* __restrict__ y, const float* __restrict__ mix,
+    const float* __restrict__ out_w, const float* __restrict__ in_w,
+    const float* __restrict__ gamma, float eps, TOut* __restrict__ normed,
+    float* __restrict__ zero, int width, int streams) {
+  __shared__ float red[16];
+  __shared__ float s_mix[HS_MAX_STREAMS * HS_MAX_STREAMS];
+  __shared__ float s_out[HS_MAX_STREAMS];
+  __shared__ float s_in[HS_MAX_STREAMS];
+  const int t = blockIdx.x;
+  const bool writes = y != nullptr;
+  const bool reads = normed != nullptr;
+  if (threadIdx.x < streams * streams && writes) s_mix[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < streams) {
+    if (writes) s_out[threadIdx.x] = out_w[threadIdx.x];
+    if (reads) s_in[threadIdx.x] = in_w[threadIdx.x];
+  }
+  __syncthreads();
+  float u[PER];
+  float sumsq = 0.f;
+  float* row = X + (int64_t)t * streams * width;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int col = threadIdx.x + i * HS_THREADS;
+    u[i] = 0.f;
+    if (col < width) {
+      float x[HS_MAX_STREAMS];
+#pragma unroll
+      for (int s = 0; s < HS_MAX_STREAMS; ++s) x[s] = s < streams ? row[(int64_t)s * width + col] : 0.f;
+      if (writes) {
+        const float yv = y[(int64_t)t * width + col];
+        float nx[HS_MAX_STREAMS];
+#pragma unroll
+        for (int to = 0; to < HS_MAX_STREAMS; ++to) {
+          float acc = 0.f;
+          if (to < streams) {
+#pragma unroll
+            for (int from = 0; from < HS_MAX_STREAMS; ++from)
+              if (from < streams) acc = fmaf(s_mix[from * streams + to], x[from], acc);
+            acc = fmaf(s_out[to], yv, acc);
+            row[(int64_t)to * width + col] = acc;
+          }
+          nx[to] = acc;
+        }
+#pragma unroll
+        for (int s = 0; s < HS_MAX_STREAMS; ++s) x[s] = nx[s];
+      }
+      if (reads) {
+        float uu = 0.f;
+#pragma unroll
+        for (int s = 0; s < HS_MAX_STREAMS; ++s)
+          if (s < streams) uu = fmaf(s_in[s], x[s], uu);
+        u[i] = uu;
+        sumsq = fmaf(uu, uu, sumsq);
+      }
+      if (zero != nullptr) zero[(int64_t)t * width + col] = 0.f;
+    }
+  }
+  if (!reads) return;
+  const float total = block_sum(sumsq, red);
+  const float inv = 1.0f / sqrtf(total / (float)width + eps);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int col = threadIdx.x + i * HS_THREADS;
+    if (col < width) normed[(int64_t)t * width + col] = from_float<TOut>(u[i] * inv * gamma[col]);
+  }
+}
+
+extern "C" int ps_hyper_step(float* x, const float* y, const float* mix, const float* out_w,
+                             const float* in_w, const float* gamma, float eps, void* normed,
+                             float* zero, int tokens, int width, int streams, int out_dtype,
+                             void* stream) {
+  PS_REQUIRE(tokens >= 0 && width > 0, "ps_hyper_step: bad sizes");
+  PS_REQUIRE(streams >= 1 && streams <= HS_MAX_STREAMS, "ps_hyper_step: %d streams, the kernel takes 1..%d",
+             streams, HS_MAX_STREAMS);
+  PS_REQUIRE(width <= HS_THREADS * 32, "ps_hyper_step: width %d above %d", width, HS_THREADS * 32);
+  PS_REQUIRE(y == nullptr || (mix != nullptr && out_w != nullptr), "ps_hyper_step: a write needs mix and out weights");
+  PS_REQUIRE(normed == nullptr || (in_w != nullptr && gamma != nullptr && eps > 0.f),
+             "ps_hyper_step: a read needs in weights, gamma and a positive eps");
+  PS_REQUIRE(out_dtype == PS_F32 || out_dtype == PS_BF16, "ps_hyper_step: unknown dtype %d", out_dtype);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+#define PS_LAUNCH_HS(TOut, PER)                                                                  \
+  hipLaunchKernelGGL((hyper_step_kernel<TOut, PER>), dim3(tokens), dim3(HS_THREADS), 0, s, x, y, \
+                     mix, out_w, in_w, gamma, eps, (TOut*)normed, zero, width, streams)
+#define PS_LAUNCH_HS_T(TOut)                         \
+  do {                                               \
+    const int per = (width + HS_THREADS - 1) / HS_THREADS; \
+    if (per <= 1) PS_LAUNCH_HS(TOut, 1);             \
+    else if (per <= 2) PS_LAUNCH_HS(TOut, 2);        \
+    else if (per <= 4) PS_LAUNCH_HS(TOut, 4);        \
+    else if (per <= 8) PS_LAUNCH_HS(TOut, 8);        \
+    else if (per <= 16) PS_LAUNCH_HS(TOut, 16);      \
+    else PS_LAUNCH_HS(TOut, 32);                     \
+  } while (0)
+  if (out_dtype == PS_F32) PS_LAUNCH_HS_T(float);
+  else PS_LAUNCH_HS_T(bf16_t);
+#undef PS_LAUNCH_HS_T
+#undef PS_LAUNCH_HS
+  PS_CHECK_LAUNCH("ps_hyper_step");
+  return 0;
+}
+
+// X[t, s, :] = e[t, :] for every copy s.
+__global__ void streams_expand_kernel(const float* __restrict__ e, float* __restrict__ X,
+                                      int width, int streams) {
+  const int t = blockIdx.x;
+  for (int col = threadIdx.x; col < width; col += blockDim.x) {
+    const float v = e[(int64_t)t * width + col];
+    for (int s = 0; s < streams; ++s) X[((int64_t)t * streams + s) * width + col] = v;
+  }
+}
+
+extern "C" int ps_streams_expand(const float* e, float* x, int tokens, int width, int streams,
+                                 void* stream) {
+  PS_REQUIRE(tokens >= 0 && width > 0 && streams > 0, "ps_streams_expand: bad sizes");
+  if (tokens == 0) return 0;
+  hipLaunchKernelGGL(streams_expand_kernel, dim3(tokens), dim3(width >= 256 ? 256 : 64), 0,
+                     (hipStream_t)stream, e, x, width, streams);
+  PS_CHECK_LAUNCH("ps_streams_expand");
+  return 0;
+}
+
+// out[r, :] = sum_s X[rows ? rows[r] : r, s, :].
+__global__ void streams_collapse_kernel(const float* __restrict__ X, const int* __restrict__ rows,
+                                        float* __restrict__ out, int width, int streams) {
+  const int r = blockIdx.x;
+  const int t = rows ? rows[r] : r;
+  for (int col = threadIdx.x; col < width; col += blockDim.x) {
+    float v = 0.f;
+    for (int s = 0; s < streams; ++s) v += X[((int64_t)t * streams + s) * width + col];
+    out[(int64_t)r * width + col] = v;
+  }
+}
+
+extern "C" int ps_streams_collapse(const float* x, const int* rows, float* out, int n_rows,
+                                   int width, int streams, void* stream) {
+  PS_REQUIRE(n_rows >= 0 && width > 0 && streams > 0, "ps_streams_collapse: bad sizes");
+  if (n_rows == 0) return 0;
+  hipLaunchKernelGGL(streams_collapse_kernel, dim3(n_rows), dim3(width >= 256 ? 256 : 64), 0,
+                     (hipStream_t)stream, x, rows, out, width, streams);
+  PS_CHECK_LAUNCH("ps_streams_collapse");
+  return 0;
+}

@@ -86,11 +86,18 @@ class Engine:
         self.max_requests = max_requests
         self.max_step_tokens = max_step_tokens
         groups, states = model.cache_requirements()
+        # A request cannot grow beyond the model's positions, nor (where no group gives pages
+        # back behind a window) beyond what the pool holds: block tables are that wide.  A model
+        # whose positions have no bound of their own (rotations) names a large number.
+        self.max_positions = self.spec.max_positions
+        if groups and not any(group.window > 0 for group in groups):
+            smallest = num_pages if isinstance(num_pages, int) else min(num_pages)
+            self.max_positions = min(self.max_positions, smallest * page_size)
         self.cache = CacheManager(groups, num_pages, page_size, max_requests, self.dtype,
-                                  self.device, states, max_positions=self.spec.max_positions)
+                                  self.device, states, max_positions=self.max_positions)
         self.views = model.cache_views(self.cache)
         self.workspace = Workspace(max_step_tokens, self.device)
-        self.table_width = -(-self.spec.max_positions // page_size)
+        self.table_width = -(-self.max_positions // page_size)
         # queries of an item with several tokens are listed in tiles, once for every tile size
         # that a mixer of the model asks for (none: no mixer wants tiles)
         self.query_tiles = tuple(getattr(model, "query_tiles", ()))
@@ -184,9 +191,9 @@ class Engine:
         than with those of 1,024, half of which they leave empty; a layout is recorded once
         more on its way to long contexts.)"""
         bound = 128
-        while bound < longest and bound < self.spec.max_positions:
+        while bound < longest and bound < self.max_positions:
             bound *= 2
-        return min(bound, self.spec.max_positions)
+        return min(bound, self.max_positions)
 
     # ------------------------------------------------------------------- step
     def _validate(self, entries):
@@ -197,7 +204,7 @@ class Engine:
         new = 0
         vocab = self.spec.vocab_size
         requests = self.cache.requests
-        max_positions = self.spec.max_positions
+        max_positions = self.max_positions
         for entry in entries:
             if entry.request_id in seen:
                 # src/model/iteration.py:61-63
@@ -237,10 +244,10 @@ class Engine:
             record = self.cache.requests.get(entry.request_id)
             have = record.length if record is not None else 0
             new += record is None
-            if have + count > self.spec.max_positions:
+            if have + count > self.max_positions:
                 # src/model/paged_decoder.py:521-522
                 raise StepError(f"request {entry.request_id!r} would reach position "
-                                f"{have + count - 1}, the model has {self.spec.max_positions}")
+                                f"{have + count - 1}, the engine takes {self.max_positions}")
             total += count
         if total > self.max_step_tokens:
             raise StepError(f"step of {total} tokens exceeds max_step_tokens={self.max_step_tokens}")
@@ -448,7 +455,7 @@ class Engine:
             page_size=self.page_size, workspace=self.workspace,
             decode_only=singles == items, max_kv_len=max_kv,
             single_tokens=views["single_tokens"], portion_tokens=views["portion_tokens"],
-            max_positions=self.spec.max_positions,
+            max_positions=self.max_positions,
             query_tiles={tile: (views[f"tile_item{tile}"], views[f"tile_q0{tile}"])
                          for tile in tile_sizes},
             token_src=views["token_src"], carried_tokens=self._tokens)

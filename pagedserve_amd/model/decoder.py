@@ -145,14 +145,34 @@ class DecoderModel:
         ``self.tokens_chosen`` says whether it did."""
         self.tokens_chosen = False
         tokens = ctx.tokens
-        h = ctx.workspace.first_rows("residual", self.spec.width, torch.float32, tokens)
-        self.embedding.forward(ctx, self.position.embedding_table(), h)
-        for call, view in zip(self.spec.schedule, views):
-            self.blocks[call.block].forward(h, ctx, view)
+        width, streams = self.spec.width, self.spec.streams
+        if streams:
+            # the stream in several copies, all equal to the embedding at the start
+            embedded = ctx.workspace.first_rows("embedded", width, torch.float32, tokens)
+            self.embedding.forward(ctx, self.position.embedding_table(), embedded)
+            h = ctx.workspace.first_rows("residual", streams * width, torch.float32, tokens)
+            kernels.streams_expand(embedded, h, tokens, width, streams)
+        else:
+            h = ctx.workspace.first_rows("residual", width, torch.float32, tokens)
+            self.embedding.forward(ctx, self.position.embedding_table(), h)
+        schedule = self.spec.schedule
+        for index, (call, view) in enumerate(zip(schedule, views)):
+            block = self.blocks[call.block]
+            block.forward(h, ctx, view)
+            # a block may leave its last write to the block that follows, if that one takes it
+            if hasattr(block, "finish"):
+                follower = self.blocks[schedule[index + 1].block] if index + 1 < len(schedule) else None
+                if not getattr(follower, "takes_stream_write", False):
+                    block.finish(h, ctx)
         wanted = logit_rows.numel()
         if wanted == 0:
             return logits_out[:0]
-        final = ctx.workspace.first_rows("final", self.spec.width, self.dtype, wanted)
+        final = ctx.workspace.first_rows("final", width, self.dtype, wanted)
+        if streams:
+            # the sum of the copies, of the wanted rows only
+            summed = ctx.workspace.first_rows("summed", width, torch.float32, wanted)
+            h = kernels.streams_collapse(h, logit_rows, summed, width, streams)
+            logit_rows = None
         normed = None
         if getattr(self.head, "accepts_pending_norm", False):
             normed = self.final_norm.pending(h, final, rows=logit_rows)

@@ -7,8 +7,8 @@ import torch
 
 from ..config.base import read_config_json
 from ..config.registry import resolve_architecture
-from ..weights.loader import load_parameters
-from ..weights.safetensors_io import write_safetensors
+from ..weights.loader import canonical_names, load_parameters
+from ..weights.safetensors_io import SafetensorsFile, write_safetensors
 from .decoder import DecoderModel
 
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
@@ -29,6 +29,10 @@ def load_model(folder, dtype="float32", device="cuda"):
     raw = read_config_json(folder)
     architecture = resolve_architecture(raw)
     config = architecture.config_class.from_dict(raw)
+    if architecture.complete_config is not None:
+        with SafetensorsFile(os.path.join(folder, "model.safetensors")) as handle:
+            stored = canonical_names(handle.names(), architecture.strip_prefixes)
+            config = architecture.complete_config(config, lambda name: tuple(handle.shape(stored[name])))
     spec = architecture.build_spec(config)
     engine_dtype = resolve_dtype(dtype)
     model = DecoderModel(spec, engine_dtype, device)

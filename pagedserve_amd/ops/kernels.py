@@ -14,8 +14,11 @@ from .library import load_library
 
 F32 = 0
 BF16 = 1
+# whether every attention kernel takes a sink (else a layer with one runs on the row-wise kernel)
+SINK_IN_ALL_KERNELS = False
+MAX_STREAMS = 8   # copies of the residual stream that ps_hyper_step takes (csrc/streams.hip)
 
-EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2, "residual": 3}
+EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2, "residual": 3, "relu2": 4}
 
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
@@ -30,7 +33,23 @@ _SIGNATURES = {
                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_attention_rowwise": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                             c_int, c_float, c_int, c_int, c_void_p],
+                             c_int, c_float, c_int, c_void_p, c_int, c_void_p],
+    "ps_hyper_step": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
+                      c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_streams_expand": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ps_streams_collapse": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ps_attention_prepare": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_int64, c_void_p,
+                             c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p,
+                             c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_head_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_gla_decay": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int,
+                     c_int, c_int, c_void_p],
+    "ps_gla_scan": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "ps_gla_output": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
+                      c_int, c_int, c_int, c_void_p],
+    "ps_softcap": [c_void_p, c_int64, c_int, c_int, c_float, c_void_p],
     "ps_attention_decode": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                             c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
@@ -629,16 +648,28 @@ def _attention_args(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, to
     return pages, kv_heads, page_size, head_dim, q_stride, out_stride, count
 
 
+def _check_sink(sink, heads):
+    """One float per head that enters the softmax's denominator as ``exp(sink[head])``, or None."""
+    if sink is None:
+        return 0
+    _check(sink, "sink", torch.float32, 1)
+    if sink.numel() != heads or not sink.is_contiguous():
+        raise KernelError(f"attention: the sink needs one float per head ({heads})")
+    return sink.data_ptr()
+
+
 def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, window=0,
-                      tok_list=None):
+                      tok_list=None, sink=None):
     """out[t, h] = softmax(q[t, h] . K * scale) V over the cached keys of t's request, for the
-    tokens in ``tok_list`` (all when it is None)."""
+    tokens in ``tok_list`` (all when it is None).  ``sink``: one float per head whose
+    exponential joins the denominator (a score that has no key and no value)."""
     pages, kv_heads, page_size, head_dim, q_stride, out_stride, count = _attention_args(
         q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list)
+    sink = _check_sink(sink, heads)
     _call("ps_attention_rowwise", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
           out.data_ptr(), out_stride, _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(),
           tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
-          float(scale), int(window), dtype_code(q.dtype), _stream())
+          float(scale), int(window), sink, dtype_code(q.dtype), _stream())
     return out
 
 
@@ -650,7 +681,7 @@ def decode_keys_per_block(head_dim: int, waves: int = 4) -> int:
 
 
 def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
-                     partial=None, window=0, tok_list=None, waves=4):
+                     partial=None, window=0, tok_list=None, waves=4, sink=None):
     """The same result as ``attention_rowwise`` by the split-KV kernel; ``partial`` is float
     scratch of ``count * heads * splits * (head_dim + 2)`` values when ``splits > 1``.
     ``tok_item=None`` says that token t is item t (row t of ``tables``), as in a step of single
@@ -686,7 +717,7 @@ def merge_linear_supported(dtype, tokens, head_dim, packed) -> bool:
 
 
 def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tables, heads, scale, splits,
-                             window=0, tok_list=None, waves=4):
+                             window=0, tok_list=None, waves=4, sink=None):
     """The per-range records of decode attention only (``partial``: float scratch of
     ``count * heads * splits * (head_dim + 2)`` values); ``attention_merge_linear`` merges them.
     ``tok_item=None``: token t is item t, as for ``attention_decode``."""
@@ -815,7 +846,7 @@ def prefill_large_tile_pays(heads, head_dim, large_tiles, max_kv_len=0) -> bool:
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
                       heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE, memo=None,
-                      shared=None):
+                      shared=None, sink=None):
     """Attention of items with several tokens, ``query_tile`` (64, 32 or 128) queries per block,
     on the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
     the tiles that see the most keys belong first.
@@ -871,7 +902,7 @@ _TILED_F32_CHECKED = False
 
 
 def attention_tiled_f32(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
-                        scale, window=0):
+                        scale, window=0, sink=None):
     """Attention of items with several tokens in true 32-bit, ``PREFILL_TILE`` queries per
     block: keys and values pass through LDS once per tile of queries instead of once per query
     (``attention_rowwise``), scores and sums are plain float arithmetic.  The tile list is the
@@ -957,7 +988,8 @@ def _sibling_call(memo, shared, key, step_key, k_pool, v_pool):
 
 
 def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_item, tile_q0,
-                    cu_tokens, kv_lens, tables, heads, scale, window=0, memo=None, shared=None):
+                    cu_tokens, kv_lens, tables, heads, scale, window=0, memo=None, shared=None,
+                    sink=None):
     """The attention of a step that mixes decoded tokens with prompt portions, in one launch:
     the tokens listed in ``tok_list`` (the step's one-token items) as ``attention_decode`` with
     one range of keys computes them, the tiles of 64 queries listed in ``tile_item`` /
@@ -1008,6 +1040,181 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
                 kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
+
+
+def _float_rows(tensor, name, rows, columns):
+    _check(tensor, name, torch.float32, 2)
+    if tensor.shape[0] < rows or tensor.shape[1] != columns or not tensor.is_contiguous():
+        raise KernelError(f"{name} must be contiguous float [>= {rows}, {columns}], got {tuple(tensor.shape)}")
+    return tensor.data_ptr()
+
+
+def _float_vector(tensor, name, count):
+    _check(tensor, name, torch.float32)
+    if tensor.numel() != count or not tensor.is_contiguous():
+        raise KernelError(f"{name} must hold {count} floats, got shape {tuple(tensor.shape)}")
+    return tensor.data_ptr()
+
+
+def hyper_step(x, tokens, width, streams, write=None, read=None, zero=None):
+    """One pass over the copies of the residual stream ``x`` (float ``[>= tokens, streams * width]``).
+
+    ``write = (y, mix, out)``: every copy becomes a mixture of the old copies plus a share of
+    the sublayer's result, ``x'_t = sum_s mix[s, t] x_s + out[t] y`` (``y``: float ``[tokens, width]``).
+    ``read = (in, gamma, eps, normed)``: ``u = sum_s in[s] x'_s`` and its RMS norm times ``gamma``
+    is written to ``normed`` (engine dtype).  ``zero``: a float ``[tokens, width]`` buffer that is
+    cleared (it may be ``y``: the next sublayer's products add into it)."""
+    _float_rows(x, "x", tokens, streams * width)
+    y = mix = out_w = in_w = gamma = normed = None
+    eps, out_code = 1.0, F32
+    if write is not None:
+        y, mix, out_w = write
+        _float_rows(y, "y", tokens, width)
+        _float_vector(mix, "mix", streams * streams)
+        _float_vector(out_w, "out weights", streams)
+    if read is not None:
+        in_w, gamma, eps, normed = read
+        _float_vector(in_w, "in weights", streams)
+        _float_vector(gamma, "gamma", width)
+        _check(normed, "normed", ndim=2)
+        if normed.shape[0] < tokens or normed.shape[1] != width or not normed.is_contiguous():
+            raise KernelError("hyper_step: normed must be contiguous [>= tokens, width]")
+        out_code = dtype_code(normed.dtype)
+    if zero is not None:
+        _float_rows(zero, "zero", tokens, width)
+    _call("ps_hyper_step", x.data_ptr(), _ptr(y), _ptr(mix), _ptr(out_w), _ptr(in_w), _ptr(gamma),
+          float(eps), _ptr(normed), _ptr(zero), tokens, width, streams, out_code, _stream())
+
+
+def streams_expand(e, x, tokens, width, streams):
+    """``x[t, s] = e[t]`` for every copy ``s``."""
+    _float_rows(e, "e", tokens, width)
+    _float_rows(x, "x", tokens, streams * width)
+    _call("ps_streams_expand", e.data_ptr(), x.data_ptr(), tokens, width, streams, _stream())
+
+
+def streams_collapse(x, rows, out, width, streams):
+    """``out[r] = sum_s x[rows[r], s]`` (all rows in order when ``rows`` is None)."""
+    _check(x, "x", torch.float32, 2)
+    if x.shape[1] != streams * width or not x.is_contiguous():
+        raise KernelError("streams_collapse: x must be contiguous [tokens, streams * width]")
+    if rows is not None:
+        _check(rows, "rows", torch.int32, 1)
+        count = rows.numel()
+    else:
+        count = x.shape[0]
+    _float_rows(out, "out", count, width)
+    _call("ps_streams_collapse", x.data_ptr(), _ptr(rows), out.data_ptr(), count, width, streams, _stream())
+    return out[:count]
+
+
+def attention_prepare(proj, columns, q_out, k_pool, v_pool, tok_item, tok_pos, tables, heads,
+                      key_dim, value_dim, q_gamma=None, k_gamma=None, eps=1e-6, freqs=None,
+                      rot_dims=0, v_first=None, v_lambda=None, v_mode=0):
+    """Norm, rotation, value mixing and cache write of an attention layer's projection
+    (``csrc/pagedserve_hip.h: ps_attention_prepare``).  ``proj``: float ``[tokens, ld]`` with
+    the query, key and value columns at ``columns = (q, k, v)``; the pools' head size is the
+    width that every head is stored with."""
+    _check(proj, "proj", torch.float32, 2)
+    ld = _rows(proj, "proj")
+    tokens = proj.shape[0]
+    pages, kv_heads, page_size, cache_dim = _check_pools(k_pool, v_pool, q_out.dtype)
+    _check(q_out, "q_out", ndim=2)
+    q_stride = _rows(q_out, "q_out")
+    if q_out.shape[0] < tokens or q_out.shape[1] != heads * cache_dim:
+        raise KernelError("attention_prepare: q_out must hold heads x cached head size per row")
+    q_col, k_col, v_col = columns
+    if max(q_col + heads * key_dim, k_col + kv_heads * key_dim, v_col + kv_heads * value_dim) > proj.shape[1]:
+        raise KernelError("attention_prepare: the projection's rows are too short for its columns")
+    _check_step_index(tok_item, tok_pos, tables, tokens)
+    if q_gamma is not None:
+        _float_vector(q_gamma, "q_gamma", heads * key_dim)
+    if k_gamma is not None:
+        _float_vector(k_gamma, "k_gamma", kv_heads * key_dim)
+    if rot_dims:
+        _float_vector(freqs, "freqs", rot_dims // 2)
+    if v_mode:
+        _check(v_first, "v_first", q_out.dtype, 2)
+        if v_first.shape[0] < tokens or v_first.shape[1] != kv_heads * value_dim or not v_first.is_contiguous():
+            raise KernelError("attention_prepare: v_first must be contiguous [>= tokens, kv_heads * value_dim]")
+    if v_mode == 2:
+        _float_vector(v_lambda, "v_lambda", 1)
+    _call("ps_attention_prepare", proj.data_ptr(), ld, q_col, k_col, v_col, q_out.data_ptr(), q_stride,
+          k_pool.data_ptr(), v_pool.data_ptr(), _ptr(q_gamma), _ptr(k_gamma), float(eps), _ptr(freqs),
+          int(rot_dims), _ptr(v_first), _ptr(v_lambda), int(v_mode), tok_item.data_ptr(),
+          tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens, heads, kv_heads, key_dim,
+          value_dim, cache_dim, page_size, pages, dtype_code(q_out.dtype), _stream())
+
+
+def head_gate(context, gate, heads, head_dim):
+    """``context[t, h, :] *= sigmoid(gate[t, h])``; ``gate``: float columns of a wider tensor."""
+    _check(context, "context", ndim=2)
+    _check(gate, "gate", torch.float32, 2)
+    tokens = context.shape[0]
+    if context.shape[1] != heads * head_dim or gate.shape[0] < tokens or gate.shape[1] != heads:
+        raise KernelError("head_gate: context [tokens, heads * head_dim] and gate [tokens, heads] needed")
+    _call("ps_head_gate", context.data_ptr(), _rows(context, "context"), gate.data_ptr(),
+          _rows(gate, "gate"), tokens, heads, head_dim, dtype_code(context.dtype), _stream())
+
+
+def gla_decay(proj, low_col, w, bias, tau, alpha):
+    """``alpha[t, c] = sigmoid(bias[c] + sum_r proj[t, low_col + r] w[c, r]) ** (1 / tau)`` in float."""
+    _check(proj, "proj", torch.float32, 2)
+    _check(w, "w", ndim=2)
+    tokens = proj.shape[0]
+    channels, rank = w.shape
+    if not w.is_contiguous() or low_col + rank > proj.shape[1]:
+        raise KernelError("gla_decay: w must be contiguous and its rank fit the projection's rows")
+    if bias is not None:
+        _float_vector(bias, "bias", channels)
+    _float_rows(alpha, "alpha", tokens, channels)
+    _call("ps_gla_decay", proj.data_ptr(), _rows(proj, "proj"), low_col, rank, w.data_ptr(), _ptr(bias),
+          float(tau), alpha.data_ptr(), tokens, channels, dtype_code(w.dtype), _stream())
+
+
+def gla_scan(proj, columns, alpha, state, out, cu_tokens, slots, heads, key_dim, value_dim, q_scale):
+    """The recurrence of gated linear attention over the step's items, token after token
+    (``csrc/pagedserve_hip.h: ps_gla_scan``); ``state``: float ``[slots, heads, key_dim, value_dim]``."""
+    _check(proj, "proj", torch.float32, 2)
+    tokens = proj.shape[0]
+    q_col, k_col, v_col = columns
+    if max(q_col + heads * key_dim, k_col + heads * key_dim, v_col + heads * value_dim) > proj.shape[1]:
+        raise KernelError("gla_scan: the projection's rows are too short for its columns")
+    _float_rows(alpha, "alpha", tokens, heads * key_dim)
+    _float_rows(out, "out", tokens, heads * value_dim)
+    _check(state, "state", torch.float32, 4)
+    if tuple(state.shape[1:]) != (heads, key_dim, value_dim) or not state.is_contiguous():
+        raise KernelError(f"gla_scan: state {tuple(state.shape)} must be [slots, {heads}, {key_dim}, {value_dim}]")
+    _check(cu_tokens, "cu_tokens", torch.int32, 1)
+    _check(slots, "slots", torch.int32, 1)
+    items = slots.numel()
+    if cu_tokens.numel() != items + 1 or not (cu_tokens.is_contiguous() and slots.is_contiguous()):
+        raise KernelError("gla_scan: cu_tokens must hold one entry more than slots")
+    _call("ps_gla_scan", proj.data_ptr(), _rows(proj, "proj"), q_col, k_col, v_col, alpha.data_ptr(),
+          state.data_ptr(), out.data_ptr(), cu_tokens.data_ptr(), slots.data_ptr(), items,
+          state.shape[0], heads, key_dim, value_dim, float(q_scale), _stream())
+
+
+def gla_output(o, weight, eps, gate, out, heads, value_dim):
+    """``out[t, h] = rms_norm(o[t, h]) * weight * silu(gate[t, h])`` over each head's values."""
+    _check(gate, "gate", torch.float32, 2)
+    tokens = gate.shape[0]
+    _float_rows(o, "o", tokens, heads * value_dim)
+    _float_vector(weight, "weight", value_dim)
+    _check(out, "out", ndim=2)
+    if gate.shape[1] != heads * value_dim or out.shape[0] < tokens or out.shape[1] != heads * value_dim:
+        raise KernelError("gla_output: gate and out must hold heads x value_dim columns")
+    _call("ps_gla_output", o.data_ptr(), weight.data_ptr(), float(eps), gate.data_ptr(), _rows(gate, "gate"),
+          out.data_ptr(), _rows(out, "out"), tokens, heads, value_dim, dtype_code(out.dtype), _stream())
+
+
+def softcap(logits, cap):
+    """``logits <- cap * tanh(logits / cap)`` in place (float rows of a possibly wider buffer)."""
+    _check(logits, "logits", torch.float32, 2)
+    if logits.shape[0]:
+        _call("ps_softcap", logits.data_ptr(), _rows(logits, "logits"), logits.shape[0], logits.shape[1],
+              float(cap), _stream())
+    return logits
 
 
 def sample(logits, inv_temperature, uniform, out):

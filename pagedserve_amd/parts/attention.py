@@ -19,6 +19,25 @@ class Attention(Mixer):
     prompt portion, a whole prompt and a decoded token are one case: every query at
     position p reads keys ``0..p`` (the last ``window`` of them) from the pages.
     ``scale`` multiplies the scores (``head_dim**-0.5`` in src/model/paged_attention.py:27).
+
+    Options, all off by default; any of them puts one launch between the projection (then
+    written in float) and the attention kernels (``kernels.attention_prepare``):
+
+    * ``value_dim``: the values' head size where it is not the keys'.  Heads are then cached
+      ``cache_dim`` wide (the larger size rounded up to 16, zeros behind), the one head size that
+      the attention kernels see; the output projection gets zero columns to match.
+    * ``qk_norm``: queries and keys are RMS-normed over the whole projection (all heads at
+      once) with a weight per column (``q_norm.gamma``, ``k_norm.gamma``) and ``norm_eps``,
+      before the rotation.
+    * ``rotary_dims`` / ``rotary_base``: the first ``rotary_dims`` dimensions of every query
+      and key head are rotated by the position, dimension 2i with 2i+1, angle ``p base^(-2i/dims)``.
+    * ``sink``: a learned number per head (``sink``) whose exponential joins the softmax's
+      denominator; it has no key and no value.
+    * ``value_mix``: ``"source"`` leaves the step's values for later layers; ``"mix"`` caches
+      ``(1 - l) v + l v_source`` with the learned ``value_mix.weight`` ``l`` and the source's
+      values of the same token.
+    * ``head_gate``: each head's output is multiplied by ``sigmoid`` of a projection of the
+      layer's input (one more row per head in the packed product, ``[q | k | v | gate]``).
     """
 
     graph_safe = True
@@ -33,35 +52,77 @@ class Attention(Mixer):
     # tiled kernel's three; ``kernels.attention_prefill`` checks them against the library's)
     query_tile = (kernels.PREFILL_TILE, kernels.PREFILL_SMALL_TILE, kernels.PREFILL_LARGE_TILE)
 
+    VALUE_MIXES = ("none", "source", "mix")
+
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
-                 window: int = 0, bias: bool = True):
+                 window: int = 0, bias: bool = True, value_dim: int = 0, qk_norm: bool = False,
+                 norm_eps: float = 1e-6, rotary_dims: int = 0, rotary_base: float = 10000.0,
+                 sink: bool = False, value_mix: str = "none", head_gate: bool = False):
         if heads % kv_heads != 0:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
         if not 0 < head_dim <= 256:
             raise ValueError(f"head_dim {head_dim} must lie in 1..256")
+        if not 0 <= value_dim <= 256:
+            raise ValueError(f"value_dim {value_dim} must lie in 1..256")
+        if value_mix not in self.VALUE_MIXES:
+            raise ValueError(f"value_mix {value_mix!r}; known: {', '.join(self.VALUE_MIXES)}")
+        if rotary_dims < 0 or rotary_dims % 2 or rotary_dims > head_dim:
+            raise ValueError(f"rotary_dims {rotary_dims} must be even and at most head_dim {head_dim}")
         self.width = width
         self.dtype = dtype
         self.heads = heads
         self.kv_heads = kv_heads
-        self.head_dim = head_dim
+        self.key_dim = head_dim
+        self.value_dim = value_dim or head_dim
         self.scale = float(scale)
         self.window = int(window)
         self.bias = bias
-        self.q_cols = heads * head_dim
-        self.kv_cols = kv_heads * head_dim
+        self.qk_norm = bool(qk_norm)
+        self.norm_eps = float(norm_eps)
+        self.rotary_dims = int(rotary_dims)
+        self.rotary_base = float(rotary_base)
+        self.has_sink = bool(sink)
+        self.value_mix = value_mix
+        self.head_gate = bool(head_gate)
+        self.prepared = (self.value_dim != self.key_dim or self.qk_norm or self.rotary_dims > 0
+                         or value_mix != "none" or self.head_gate)
+        # the head size that the cache and the attention kernels see
+        self.head_dim = head_dim
+        if self.value_dim != self.key_dim:
+            self.head_dim = -(-max(self.key_dim, self.value_dim) // 16) * 16
+        elif self.prepared and head_dim % 2:
+            self.head_dim = head_dim + 1
+        self.q_cols = heads * self.head_dim         # columns of the queries and of the context
+        self.kv_cols = kv_heads * self.head_dim
+        self.sink = None
         self.position = None
         # what ``kernels.linear`` keeps per call site and step shape (its ``memo``), per workspace
         self._memo_qkv, self._memo_out, self._memo_attention = {}, {}, {}
 
+    def _projection_columns(self):
+        """First column of the queries, keys, values and gates in the packed product, and its width."""
+        q_col = 0
+        k_col = q_col + self.heads * self.key_dim
+        v_col = k_col + self.kv_heads * self.key_dim
+        gate_col = v_col + self.kv_heads * self.value_dim
+        return q_col, k_col, v_col, gate_col, gate_col + (self.heads if self.head_gate else 0)
+
     def parameters(self):
-        total = self.q_cols + 2 * self.kv_cols
+        total = self._projection_columns()[4]
         params = {
             "qkv.weight": ParamSpec((total, self.width), MATRIX),
-            "out.weight": ParamSpec((self.width, self.q_cols), MATRIX),
+            "out.weight": ParamSpec((self.width, self.heads * self.value_dim), MATRIX),
         }
         if self.bias:
             params["qkv.bias"] = ParamSpec((total,), VECTOR)
             params["out.bias"] = ParamSpec((self.width,), VECTOR)
+        if self.qk_norm:
+            params["q_norm.gamma"] = ParamSpec((self.heads * self.key_dim,), VECTOR)
+            params["k_norm.gamma"] = ParamSpec((self.kv_heads * self.key_dim,), VECTOR)
+        if self.has_sink:
+            params["sink"] = ParamSpec((self.heads,), VECTOR)
+        if self.value_mix == "mix":
+            params["value_mix.weight"] = ParamSpec((), VECTOR)
         return params
 
     def bind(self, tensors):
@@ -69,6 +130,22 @@ class Attention(Mixer):
         self.out_weight = tensors["out.weight"]
         self.qkv_bias = tensors.get("qkv.bias")
         self.out_bias = tensors.get("out.bias")
+        self.q_gamma = tensors.get("q_norm.gamma")
+        self.k_gamma = tensors.get("k_norm.gamma")
+        self.sink = tensors.get("sink")
+        self.mix_weight = tensors["value_mix.weight"].reshape(1) if self.value_mix == "mix" else None
+        if self.head_dim != self.value_dim:
+            # heads are cached wider than the values: the context has zero columns there, and
+            # the output projection gets zero columns to match
+            padded = self.out_weight.new_zeros((self.width, self.heads, self.head_dim))
+            padded[:, :, :self.value_dim] = self.out_weight.view(self.width, self.heads, self.value_dim)
+            self.out_weight = padded.view(self.width, self.q_cols)
+        self.freqs = None
+        if self.rotary_dims:
+            # base^(-2i/dims), worked out in 64-bit and rounded once; the angle is float(p) * f
+            steps = torch.arange(self.rotary_dims // 2, dtype=torch.float64)
+            self.freqs = torch.pow(torch.tensor(self.rotary_base, dtype=torch.float64),
+                                   -2.0 * steps / self.rotary_dims).to(torch.float32).to(self.out_weight.device)
         # copies in the layout that the products of few rows (decode steps) read fastest
         self.qkv_packed = kernels.pack_decode_weight(self.qkv_weight)
         self.out_packed = kernels.pack_decode_weight(self.out_weight)
@@ -79,13 +156,59 @@ class Attention(Mixer):
     def cache_spec(self):
         return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
 
+    def _project_prepared(self, x, ctx, cache, tables):
+        """Projection in float, then norm, rotation, value mixing and cache write in one launch;
+        returns the queries (engine dtype, heads ``head_dim`` wide) and the gates' columns."""
+        if not cache.writes:
+            raise NotImplementedError("an attention layer with prepared queries and keys writes its own cache entry")
+        tokens = ctx.tokens
+        q_col, k_col, v_col, gate_col, total = self._projection_columns()
+        proj = ctx.workspace.first_rows("attn_proj", total, torch.float32, tokens)
+        kernels.linear(x, self.qkv_weight, self.qkv_bias, proj, packed=self.qkv_packed,
+                       memo=site_memo(self._memo_qkv, ctx.workspace), shared=ctx.shared_calls)
+        q = ctx.workspace.first_rows("attn_q", self.q_cols, self.dtype, tokens)
+        v_first = None
+        if self.value_mix != "none":
+            v_first = ctx.workspace.first_rows("values_source", self.kv_heads * self.value_dim,
+                                               self.dtype, tokens)
+        kernels.attention_prepare(
+            proj, (q_col, k_col, v_col), q, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions,
+            tables, self.heads, self.key_dim, self.value_dim, q_gamma=self.q_gamma,
+            k_gamma=self.k_gamma, eps=self.norm_eps, freqs=self.freqs, rot_dims=self.rotary_dims,
+            v_first=v_first, v_lambda=self.mix_weight,
+            v_mode=self.VALUE_MIXES.index(self.value_mix))
+        return q, (proj[:, gate_col:gate_col + self.heads] if self.head_gate else None)
+
+    def _project_out(self, context, gates, residual, ctx):
+        if gates is not None:
+            kernels.head_gate(context, gates, self.heads, self.head_dim)
+        kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
+                       packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace),
+                       shared=ctx.shared_calls)
+
     def forward(self, x, residual, ctx, cache):
+        tokens = ctx.tokens
+        tables = ctx.tables[cache.group]
+        gates = None
+        sink = self.sink
+        if self.prepared:
+            q, gates = self._project_prepared(x, ctx, cache, tables)
+        else:
+            q = self._project_plain(x, ctx, cache, tables)
+        context = ctx.workspace.first_rows("attn", self.q_cols, self.dtype, tokens)
+        if sink is not None and not kernels.SINK_IN_ALL_KERNELS:
+            kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
+                                      ctx.positions, tables, self.heads, self.scale, self.window,
+                                      sink=sink)
+            return self._project_out(context, gates, residual, ctx)
+        return self._attend(q, context, gates, residual, ctx, cache, tables)
+
+    def _project_plain(self, x, ctx, cache, tables):
         tokens = ctx.tokens
         total = self.q_cols + 2 * self.kv_cols
         # (the step's rows and their three column views, made once per row count for all layers)
         qkv, q, k, v = ctx.workspace.column_views("qkv", total, self.dtype, tokens,
                                                   (self.q_cols, self.kv_cols, self.kv_cols))
-        tables = ctx.tables[cache.group]
         rotates = self.position is not None and self.position.transforms_qk
         if cache.writes and not rotates:
             # keys and values go to their pages from the product's own epilogue
@@ -103,15 +226,19 @@ class Attention(Mixer):
             if cache.writes:
                 kernels.kv_write(k, v, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions,
                                  tables)
-        context = ctx.workspace.first_rows("attn", self.q_cols, self.dtype, tokens)
+        return q
+
+    def _attend(self, q, context, gates, residual, ctx, cache, tables):
+        tokens = ctx.tokens
+        sink = self.sink
         singles = ctx.single_tokens.numel() if ctx.single_tokens is not None else 0
         if not kernels.decode_supported(self.head_dim):
             # a head size that the split-KV kernel does not take: every token, decoded ones
             # too, goes to the kernel that takes all sizes
             singles = 0
         merged_splits = 0
-        if singles == tokens and kernels.merge_linear_supported(self.dtype, tokens, self.head_dim,
-                                                                 self.out_packed):
+        if gates is None and singles == tokens and kernels.merge_linear_supported(
+                self.dtype, tokens, self.head_dim, self.out_packed):
             merged_splits = self._merged_splits(singles, ctx.max_kv_len)
         if merged_splits:
             # a decode step of few tokens over long contexts: the key ranges are merged inside
@@ -120,7 +247,7 @@ class Attention(Mixer):
             partial = self._range_records(ctx)
             kernels.attention_decode_partial(q, cache.k_pool, cache.v_pool, partial, ctx.tok_item,
                                              ctx.positions, tables, self.heads, self.scale, splits,
-                                             window=self.window, waves=4)
+                                             window=self.window, waves=4, sink=sink)
             kernels.attention_merge_linear(partial, singles, self.heads, self.head_dim, splits,
                                            self.out_weight, self.out_packed, self.out_bias, residual)
             return
@@ -132,11 +259,8 @@ class Attention(Mixer):
                                     ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
                                     ctx.kv_lens, tables, self.heads, self.scale, self.window,
                                     memo=site_memo(self._memo_attention, ctx.workspace),
-                                    shared=ctx.shared_calls)
-            kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
-                           packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace),
-                       shared=ctx.shared_calls)
-            return
+                                    shared=ctx.shared_calls, sink=sink)
+            return self._project_out(context, gates, residual, ctx)
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
             # still fill the chip
@@ -156,7 +280,8 @@ class Attention(Mixer):
                                      None if direct else ctx.tok_item,
                                      ctx.positions, tables, self.heads, self.scale, splits,
                                      partial=partial, window=self.window, waves=waves,
-                                     tok_list=None if singles == tokens else ctx.single_tokens)
+                                     tok_list=None if singles == tokens else ctx.single_tokens,
+                                     sink=sink)
         whole = singles == 0
         if tiled:
             size = kernels.PREFILL_TILE
@@ -174,7 +299,7 @@ class Attention(Mixer):
                                       self.heads, self.scale, self.window,
                                       max_kv_len=ctx.max_kv_len, query_tile=size,
                                       memo=site_memo(self._memo_attention, ctx.workspace),
-                                      shared=ctx.shared_calls)
+                                      shared=ctx.shared_calls, sink=sink)
         elif singles < tokens and kernels.tiled_f32_supported(self.dtype, self.head_dim):
             # 32-bit: tiles of queries too, on plain float arithmetic.  The tiles hold the items
             # of several tokens; one-token items that the split-KV kernel did not take (a head
@@ -183,12 +308,12 @@ class Attention(Mixer):
             if tile_item.numel():
                 kernels.attention_tiled_f32(q, cache.k_pool, cache.v_pool, context, tile_item, tile_q0,
                                             ctx.cu_tokens, ctx.kv_lens, tables, self.heads, self.scale,
-                                            self.window)
+                                            self.window, sink=sink)
             if not singles and ctx.single_tokens is not None and ctx.single_tokens.numel():
                 kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                           ctx.positions, tables, self.heads, self.scale, self.window,
                                           tok_list=None if ctx.single_tokens.numel() == tokens
-                                          else ctx.single_tokens)
+                                          else ctx.single_tokens, sink=sink)
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,

@@ -6,6 +6,9 @@ which order they run; ``mixer`` is the part whose ``cache_spec`` decides what th
 entry holds.  The model builds the parts that the block's spec names and hands them
 over as a dict; an arrangement with another number of parts declares other roles."""
 
+import torch
+
+from ..ops import kernels
 from .registry import register_arrangement
 
 
@@ -46,3 +49,86 @@ class PreNormBlock:
         self.mixer.forward(self._normed(self.norm1, self.mixer, h, ctx), h, ctx, cache)
         self.feed_forward.forward(self._normed(self.norm2, self.feed_forward, h, ctx), h, ctx)
         return h
+
+
+@register_arrangement("pre_norm_mixer")
+class PreNormMixerBlock(PreNormBlock):
+    """``h += mixer(norm1(h))`` alone: a layer without a feed-forward."""
+
+    roles = {"norm1": "norm", "mixer": "mixer"}
+
+    def __init__(self, width, dtype, parts):
+        self.width = width
+        self.dtype = dtype
+        self._parts = dict(parts)
+        self.norm1 = parts["norm1"]
+        self.mixer = parts["mixer"]
+
+    def forward(self, h, ctx, cache):
+        self.mixer.forward(self._normed(self.norm1, self.mixer, h, ctx), h, ctx, cache)
+        return h
+
+
+_STREAM_WRITE = "stream_write"   # key of ``ctx.extra``: a sublayer's result that is not written back yet
+
+
+@register_arrangement("hyper_connected")
+class HyperConnectedBlock:
+    """A pre-norm layer over a residual stream of several copies (``h`` is ``[T, streams *
+    width]``): each sublayer reads a weighted sum of the copies through its norm and its result
+    is mixed back into all of them (``parts/connection.py``).  Writing a result back and
+    reading for the next sublayer is one launch; the last write of a block is left to the next
+    block's first launch (``ctx.extra``), or to ``finish``."""
+
+    roles = {"connect1": "connection", "norm1": "norm", "mixer": "mixer",
+             "connect2": "connection", "norm2": "norm", "feed_forward": "feed_forward"}
+    takes_stream_write = True
+
+    def __init__(self, width, dtype, parts):
+        self.width = width
+        self.dtype = dtype
+        self._parts = dict(parts)
+        self.mixer = parts["mixer"]
+        self.sublayers = [(parts["connect1"], parts["norm1"], self.mixer)]
+        if "feed_forward" in parts:
+            self.sublayers.append((parts["connect2"], parts["norm2"], parts["feed_forward"]))
+        self.streams = parts["connect1"].streams
+
+    @property
+    def graph_safe(self):
+        return all(getattr(part, "graph_safe", False) for part in self._parts.values())
+
+    def parts(self):
+        return dict(self._parts)
+
+    def forward(self, h, ctx, cache):
+        tokens = ctx.tokens
+        normed = ctx.workspace.first_rows("normed", self.width, self.dtype, tokens)
+        # the sublayers' last products add into y, which every launch below leaves cleared
+        y = ctx.workspace.first_rows("sublayer", self.width, torch.float32, tokens)
+        if ctx.extra is None:
+            ctx.extra = {}
+        write = ctx.extra.pop(_STREAM_WRITE, None)
+        for connection, norm, part in self.sublayers:
+            kernels.hyper_step(h, tokens, self.width, self.streams, write=write,
+                               read=connection.read_of(norm, normed), zero=y)
+            if part is self.mixer:
+                part.forward(normed, y, ctx, cache)
+            else:
+                part.forward(normed, y, ctx)
+            write = connection.write_of(y)
+        ctx.extra[_STREAM_WRITE] = write
+        return h
+
+    def finish(self, h, ctx):
+        """Write back what the last sublayer left (no block follows that would)."""
+        write = ctx.extra.pop(_STREAM_WRITE, None) if ctx.extra else None
+        if write is not None:
+            kernels.hyper_step(h, ctx.tokens, self.width, self.streams, write=write)
+
+
+@register_arrangement("hyper_connected_mixer")
+class HyperConnectedMixerBlock(HyperConnectedBlock):
+    """The same with a mixer only."""
+
+    roles = {"connect1": "connection", "norm1": "norm", "mixer": "mixer"}

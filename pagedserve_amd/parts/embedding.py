@@ -31,11 +31,16 @@ class TokenLookup(Embedding):
 @register_head("linear")
 class LinearHead(Head):
     """``logits = f W^T (+ b)`` in float.  Tied: ``W`` is the token table itself, not a copy,
-    and there is no bias (src/model/paged_decoder.py:295-301,605)."""
+    and there is no bias (src/model/paged_decoder.py:295-301,605).  ``softcap = c > 0``:
+    ``logits <- c tanh(logits / c)`` afterwards (monotonic: the most likely token stays)."""
 
     graph_safe = True
 
-    def __init__(self, width: int, dtype, vocab_size: int, tied: bool = True, bias: bool = False):
+    def __init__(self, width: int, dtype, vocab_size: int, tied: bool = True, bias: bool = False,
+                 softcap: float = 0.0):
+        if softcap < 0:
+            raise ValueError("a logit cap must be positive (0: none)")
+        self.softcap = float(softcap)
         if tied and bias:
             raise ValueError("a head tied to the token table has no bias of its own")
         self.width = width
@@ -67,7 +72,10 @@ class LinearHead(Head):
     def forward(self, x, logits, choose=None):
         if choose is None:
             kernels.linear(x, self.weight, self.bias_vector, logits, packed=self.packed)
-            return False
-        _, chosen = kernels.linear(x, self.weight, self.bias_vector, logits, packed=self.packed,
-                                   choose=choose)
+            chosen = False
+        else:
+            _, chosen = kernels.linear(x, self.weight, self.bias_vector, logits, packed=self.packed,
+                                       choose=choose)
+        if self.softcap:
+            kernels.softcap(logits, self.softcap)
         return chosen

@@ -5,7 +5,7 @@ from ..weights.loader import MATRIX, VECTOR, ParamSpec
 from .base import FeedForward, site_memo
 from .registry import register_feed_forward
 
-ACTIVATIONS = ("gelu_tanh", "gelu_erf")
+ACTIVATIONS = ("gelu_tanh", "gelu_erf", "relu2")
 
 
 @register_feed_forward("dense")

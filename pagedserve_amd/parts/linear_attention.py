@@ -1,0 +1,96 @@
+"""Recurrent mixers whose state is a matrix per head."""
+
+import torch
+
+from ..ops import kernels
+from ..weights.loader import MATRIX, VECTOR, ParamSpec
+from .base import Mixer, SlotStateSpec, site_memo
+from .registry import register_mixer
+
+
+@register_mixer("gated_linear_attention")
+class GatedLinearAttention(Mixer):
+    """Linear attention with a decay per key channel.  With ``h`` the layer's input:
+
+        q = W_q h * key_dim^(-1/2),  k = W_k h,  v = W_v h          (heads x key_dim / value_dim)
+        alpha = sigmoid(W_a2 (W_a1 h) + b)^(1 / tau)                (heads x key_dim)
+        S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t   (per head)
+        out = W_o (rms_norm_per_head(o) * w_norm * silu(W_g h))
+
+    The state ``S`` (float, ``[heads, key_dim, value_dim]``) lives in the request's slot,
+    starts at zero and is carried from step to step.  One packed product gives
+    ``[q | k | v | gate | low-rank decay input]`` in float; the decays, the recurrence and the
+    per-head norm are 32-bit (``csrc/gla.hip``)."""
+
+    graph_safe = True
+
+    accepts_pending_norm = True
+
+    def __init__(self, width: int, dtype, heads: int, key_dim: int, value_dim: int, decay_rank: int,
+                 tau: float, norm_eps: float):
+        if not 0 < key_dim <= 256:
+            raise ValueError(f"key_dim {key_dim} must lie in 1..256")
+        if tau <= 0:
+            raise ValueError("tau must be positive")
+        self.width = width
+        self.dtype = dtype
+        self.heads = heads
+        self.key_dim = key_dim
+        self.value_dim = value_dim
+        self.decay_rank = decay_rank
+        self.tau = float(tau)
+        self.norm_eps = float(norm_eps)
+        self.k_cols = heads * key_dim
+        self.v_cols = heads * value_dim
+        self._memo_in, self._memo_out = {}, {}
+
+    def _columns(self):
+        q_col = 0
+        k_col = q_col + self.k_cols
+        v_col = k_col + self.k_cols
+        gate_col = v_col + self.v_cols
+        low_col = gate_col + self.v_cols
+        return q_col, k_col, v_col, gate_col, low_col, low_col + self.decay_rank
+
+    def parameters(self):
+        total = self._columns()[5]
+        return {
+            "in.weight": ParamSpec((total, self.width), MATRIX),
+            "decay.weight": ParamSpec((self.k_cols, self.decay_rank), MATRIX),
+            "decay.bias": ParamSpec((self.k_cols,), VECTOR),
+            "norm.gamma": ParamSpec((self.value_dim,), VECTOR),
+            "out.weight": ParamSpec((self.width, self.v_cols), MATRIX),
+        }
+
+    def bind(self, tensors):
+        self.in_weight = tensors["in.weight"]
+        self.decay_weight = tensors["decay.weight"]
+        self.decay_bias = tensors["decay.bias"]
+        self.norm_gamma = tensors["norm.gamma"]
+        self.out_weight = tensors["out.weight"]
+        self.in_packed = kernels.pack_decode_weight(self.in_weight)
+        self.out_packed = kernels.pack_decode_weight(self.out_weight)
+        self._memo_in.clear()
+        self._memo_out.clear()
+
+    def cache_spec(self):
+        return SlotStateSpec((self.heads, self.key_dim, self.value_dim), torch.float32)
+
+    def forward(self, x, residual, ctx, cache):
+        tokens = ctx.tokens
+        q_col, k_col, v_col, gate_col, low_col, total = self._columns()
+        workspace = ctx.workspace
+        proj = workspace.first_rows("gla_proj", total, torch.float32, tokens)
+        kernels.linear(x, self.in_weight, None, proj, packed=self.in_packed,
+                       memo=site_memo(self._memo_in, workspace), shared=ctx.shared_calls)
+        alpha = workspace.first_rows("gla_decay", self.k_cols, torch.float32, tokens)
+        kernels.gla_decay(proj, low_col, self.decay_weight, self.decay_bias, self.tau, alpha)
+        raw = workspace.first_rows("gla_raw", self.v_cols, torch.float32, tokens)
+        kernels.gla_scan(proj, (q_col, k_col, v_col), alpha, cache.state, raw, ctx.cu_tokens,
+                         ctx.slots, self.heads, self.key_dim, self.value_dim, self.key_dim ** -0.5)
+        gated = workspace.first_rows("gla_out", self.v_cols, self.dtype, tokens)
+        kernels.gla_output(raw, self.norm_gamma, self.norm_eps, proj[:, gate_col:gate_col + self.v_cols],
+                           gated, self.heads, self.value_dim)
+        kernels.linear(gated, self.out_weight, None, residual, epilogue="residual",
+                       packed=self.out_packed, memo=site_memo(self._memo_out, workspace),
+                       shared=ctx.shared_calls)

@@ -30,17 +30,23 @@ class LayerNorm(Norm):
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
-    """h / sqrt(mean(h^2) + eps) * gamma.  Not used by GPT-2; the kernel's second mode."""
+    """h / sqrt(mean(h^2) + eps) * (offset + gamma): the kernel's second mode.  ``offset`` is
+    1 for checkpoints that store the scale around zero; it is added once, in float, when the
+    weights are bound."""
 
     graph_safe = True
 
-    def __init__(self, width: int, dtype, eps: float):
+    def __init__(self, width: int, dtype, eps: float, offset: float = 0.0):
         self.width = width
         self.dtype = dtype
         self.eps = float(eps)
+        self.offset = float(offset)
 
     def parameters(self):
         return {"gamma": ParamSpec((self.width,), VECTOR)}
+
+    def bind(self, tensors):
+        self.gamma = tensors["gamma"] + self.offset if self.offset else tensors["gamma"]
 
     def forward(self, h, out, rows=None):
         return kernels.norm(h, self.gamma, None, self.eps, out, rows=rows, rms=True)

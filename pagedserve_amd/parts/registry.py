@@ -10,9 +10,10 @@ POSITIONS: Dict[str, Callable] = {}
 ARRANGEMENTS: Dict[str, Callable] = {}
 EMBEDDINGS: Dict[str, Callable] = {}
 HEADS: Dict[str, Callable] = {}
+CONNECTIONS: Dict[str, Callable] = {}
 
 # role of a block's named part -> the registry its kind is looked up in
-ROLES = {"norm": NORMS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS}
+ROLES = {"norm": NORMS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS, "connection": CONNECTIONS}
 
 
 def _register(table, what):
@@ -33,6 +34,7 @@ register_position = _register(POSITIONS, "position encoding")
 register_arrangement = _register(ARRANGEMENTS, "block arrangement")
 register_embedding = _register(EMBEDDINGS, "embedding")
 register_head = _register(HEADS, "output head")
+register_connection = _register(CONNECTIONS, "stream connection")
 
 
 def build_part(table, what, spec, **common):

@@ -61,6 +61,8 @@ class WeightSource:
         they cannot be joined."""
         shapes = [tuple(reversed(shape)) if self.transpose else tuple(shape) for shape in stored_shapes]
         first = list(shapes[0])
+        if len(shapes) == 1 and self.rows is None:
+            return tuple(first)      # (a single tensor as it is, a scalar included)
         if not 0 <= self.axis < len(first):
             return None
         for shape in shapes[1:]:
