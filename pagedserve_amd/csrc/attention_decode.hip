@@ -61,7 +61,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
                          const int* tok_item, const int* tok_pos, const int* tables,
                          int table_width, int count, int heads, int kv_heads, int head_dim,
                          int page_size, int num_pages, float scale, int window, int splits,
-                         int waves, hipStream_t s) {
+                         int waves, const float* sink, hipStream_t s) {
   int page_shift = -1;
   if ((page_size & (page_size - 1)) == 0) {
     page_shift = 0;
@@ -74,7 +74,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
                      (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,         \
                      out_stride, partial, tok_list, tok_item, tok_pos, tables, table_width,      \
                      heads, kv_heads, head_dim, page_size, page_shift, num_pages,                \
-                     scale * 1.4426950408889634f, window, splits)
+                     scale * 1.4426950408889634f, window, splits, sink)
   // more blocks than compute units: the step is bound by memory bandwidth, not by one round trip
   const bool streaming = sizeof(T) == 2 && (int64_t)count * heads * splits > ps_compute_units();
 #define PS_LAUNCH_ADW(LPK, WAVES)          \
@@ -196,10 +196,10 @@ extern "C" int ps_attention_decode_static(const void* q, int64_t q_stride, const
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, nullptr, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, nullptr, s);
 }
 
 // The partial records only (see pagedserve_hip.h).
@@ -210,7 +210,7 @@ extern "C" int ps_attention_decode_partial(const void* q, int64_t q_stride, cons
                                            const int* tables, int table_width, int count,
                                            int heads, int kv_heads, int head_dim, int page_size,
                                            int num_pages, float scale, int window, int splits,
-                                           int waves, int dtype, void* stream) {
+                                           int waves, const float* sink, int dtype, void* stream) {
   if (check_decode_sizes("ps_attention_decode_partial", count, heads, kv_heads, head_dim,
                          page_size, num_pages, table_width, window, splits, waves, dtype))
     return 1;
@@ -222,10 +222,10 @@ extern "C" int ps_attention_decode_partial(const void* q, int64_t q_stride, cons
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
 }
 
 extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool,
@@ -234,7 +234,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
                                    const int* tok_item, const int* tok_pos, const int* tables,
                                    int table_width, int count, int heads, int kv_heads,
                                    int head_dim, int page_size, int num_pages, float scale,
-                                   int window, int splits, int waves, int dtype, void* stream) {
+                                   int window, int splits, int waves, const float* sink, int dtype,
+                                   void* stream) {
   if (check_decode_sizes("ps_attention_decode", count, heads, kv_heads, head_dim, page_size,
                          num_pages, table_width, window, splits, waves, dtype))
     return 1;
@@ -250,8 +251,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
 }

@@ -101,7 +101,8 @@ __device__ __forceinline__ void attention_decode_block(
     float* __restrict__ partial, const int* __restrict__ tok_list,
     const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
-    int page_size, int page_shift, int num_pages, float scale_log2, int window, int splits) {
+    int page_size, int page_shift, int num_pages, float scale_log2, int window, int splits,
+    const float* __restrict__ sink) {
   constexpr int GROUPS = 64 / LPK;               // keys per wave load
   constexpr int KEYS_PER_WAVE = GROUPS * AD_UNROLL;
   float (&s_acc)[AD_WAVES][256] = lds.acc;
@@ -143,6 +144,11 @@ __device__ __forceinline__ void attention_decode_block(
                      : 0.f;
 
   float m = -INFINITY, l = 0.f;
+  if (sink != nullptr && split == 0 && wave == 0 && group == 0) {
+    // a score without key or value (not scaled): it starts the denominator of one lane group
+    m = sink[head] * 1.4426950408889634f;
+    l = 1.f;
+  }
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   for (int base = range_begin + wave * KEYS_PER_WAVE; base < range_end;
@@ -276,11 +282,12 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     float* __restrict__ partial, const int* __restrict__ tok_list,
     const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
-    int page_size, int page_shift, int num_pages, float scale_log2, int window, int splits) {
+    int page_size, int page_shift, int num_pages, float scale_log2, int window, int splits,
+    const float* __restrict__ sink) {
   __shared__ DecodeLds<AD_WAVES> lds;
   attention_decode_block<T, LPK, AD_WAVES, AD_UNROLL, NT>(
       lds, blockIdx.x, blockIdx.y, blockIdx.z, q, q_stride, k_pool, v_pool, out, out_stride, partial,
       tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads, head_dim, page_size,
-      page_shift, num_pages, scale_log2, window, splits);
+      page_shift, num_pages, scale_log2, window, splits, sink);
 }
 

@@ -49,7 +49,7 @@ __device__ __forceinline__ void attention_prefill_block(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ cu_tokens, const int* __restrict__ kv_lens,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int page_size,
-    int page_shift, int num_pages, float scale, int window) {
+    int page_shift, int num_pages, float scale, int window, const float* __restrict__ sink) {
   constexpr int HD = NDB * 16;
   constexpr int ROW = HD * 2;                    // bytes of one key in a tile
   constexpr int CH = HD / 8;                     // 16-byte pieces per row
@@ -195,6 +195,11 @@ __device__ __forceinline__ void attention_prefill_block(
   // every exponential is one v_exp_f32; probabilities are rounded to bfloat16 right after.
   const float scale_log2 = scale * 1.4426950408889634f;
   float m = -INFINITY, l = 0.f;
+  if (sink != nullptr && wave_k == 0) {
+    // a score without key or value: it starts the denominator of the wave with the first keys
+    m = sink[head] * 1.4426950408889634f;
+    l = 1.f;
+  }
   f32x16 acc[NDB32];
 #pragma unroll
   for (int db = 0; db < NDB32; ++db)
@@ -483,11 +488,11 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ cu_tokens, const int* __restrict__ kv_lens,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int page_size,
-    int page_shift, int num_pages, float scale, int window) {
+    int page_shift, int num_pages, float scale, int window, const float* __restrict__ sink) {
   __shared__ PrefillLds<NDB, KS, QW, KR> lds;
   attention_prefill_block<NDB, KS, QW, KR>(lds, blockIdx.x, blockIdx.y, q, q_stride, k_pool, v_pool, out,
                                            out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,
                                            table_width, heads, kv_heads, page_size, page_shift,
-                                           num_pages, scale, window);
+                                           num_pages, scale, window, sink);
 }
 

@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ cu_tokens, const int* __restrict__ kv_lens,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
-    int page_size, int num_pages, float scale, int window) {
+    int page_size, int num_pages, float scale, int window, const float* __restrict__ sink) {
   constexpr int STRIDE = 64 * DV + 4;   // floats from row to row of q, k and v in LDS
   __shared__ __attribute__((aligned(16))) float s_q[AF_TILE * STRIDE];
   __shared__ __attribute__((aligned(16))) float s_k[AF_TILE * STRIDE];
@@ -78,8 +78,9 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
   float4 acc[DV][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    run_max[i] = -INFINITY;
-    run_sum[i] = 0.f;
+    // (a sink is a score without key or value: it starts the denominator)
+    run_max[i] = sink ? sink[head] : -INFINITY;
+    run_sum[i] = sink ? 1.f : 0.f;
 #pragma unroll
     for (int v = 0; v < DV; ++v) acc[v][i] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
@@ -233,7 +234,7 @@ extern "C" int ps_attention_tiled_f32(const void* q, int64_t q_stride, const voi
                                       const int* cu_tokens, const int* kv_lens, const int* tables,
                                       int table_width, int heads, int kv_heads, int head_dim,
                                       int page_size, int num_pages, float scale, int window,
-                                      void* stream) {
+                                      const float* sink, void* stream) {
   PS_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_tiled_f32: bad sizes");
@@ -255,7 +256,7 @@ extern "C" int ps_attention_tiled_f32(const void* q, int64_t q_stride, const voi
   hipLaunchKernelGGL(attention_tiled_f32_kernel<DV>, dim3((unsigned)blocks), dim3(256), 0, s,     \
                      (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,       \
                      (float*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,     \
-                     table_width, heads, kv_heads, head_dim, page_size, num_pages, scale, window)
+                     table_width, heads, kv_heads, head_dim, page_size, num_pages, scale, window, sink)
   if (head_dim <= 64) {
     PS_LAUNCH_AF(1);
   } else {

@@ -133,7 +133,7 @@ int ps_attention_tiled_f32(const void* q, int64_t q_stride, const void* k_pool, 
                            void* out, int64_t out_stride, const int* tile_item, const int* tile_q0,
                            int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                            int table_width, int heads, int kv_heads, int head_dim, int page_size,
-                           int num_pages, float scale, int window, void* stream);
+                           int num_pages, float scale, int window, const float* sink, void* stream);
 
 // The same result for single queries, with each token's keys cut into `splits` ranges that
 // run as separate blocks of `waves` (4 or 16) waves; `partial` is scratch of
@@ -146,7 +146,7 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
                         const int* tok_list, const int* tok_item, const int* tok_pos,
                         const int* tables, int table_width, int count, int heads, int kv_heads,
                         int head_dim, int page_size, int num_pages, float scale, int window,
-                        int splits, int waves, int dtype, void* stream);
+                        int splits, int waves, const float* sink, int dtype, void* stream);
 
 // Only the records of ps_attention_decode: (unnormalised sum of values [head_dim], maximum in
 // units of log 2, sum) per (token, head, range) at partial[((n * heads + head) * splits + s) *
@@ -156,8 +156,8 @@ int ps_attention_decode_partial(const void* q, int64_t q_stride, const void* k_p
                                 const int* tok_list, const int* tok_item, const int* tok_pos,
                                 const int* tables, int table_width, int count, int heads,
                                 int kv_heads, int head_dim, int page_size, int num_pages,
-                                float scale, int window, int splits, int waves, int dtype,
-                                void* stream);
+                                float scale, int window, int splits, int waves, const float* sink,
+                                int dtype, void* stream);
 
 // The merge of those records inside the output projection, for up to 16 tokens and head sizes
 // that are multiples of 64 (bfloat16 weights in their packed copy, n output columns,
@@ -203,7 +203,7 @@ int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, co
                          int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                          int table_width, int heads, int kv_heads, int head_dim, int page_size,
                          int num_pages, float scale, int window, int max_kv_len, int query_tile,
-                         int dtype, void* stream);
+                         const float* sink, int dtype, void* stream);
 
 // Both of the above in one launch, for a step that has items of one token (tok_list lists the
 // `singles` tokens; tok_item and tok_pos are indexed by token as in ps_attention_decode, which
@@ -217,8 +217,8 @@ int ps_attention_mixed(const void* q, int64_t q_stride, const void* k_pool, cons
                        const int* tok_item, const int* tok_pos, const int* tile_item,
                        const int* tile_q0, int tiles, const int* cu_tokens, const int* kv_lens,
                        const int* tables, int table_width, int heads, int kv_heads, int head_dim,
-                       int page_size, int num_pages, float scale, int window, int dtype,
-                       void* stream);
+                       int page_size, int num_pages, float scale, int window, const float* sink,
+                       int dtype, void* stream);
 
 // The constants of that kernel that a caller builds its index arrays by: queries per tile (of
 // the two sizes), and the widest block table (entries per item) that it takes.

@@ -15,7 +15,7 @@ from .library import load_library
 F32 = 0
 BF16 = 1
 # whether every attention kernel takes a sink (else a layer with one runs on the row-wise kernel)
-SINK_IN_ALL_KERNELS = False
+SINK_IN_ALL_KERNELS = True
 MAX_STREAMS = 8   # copies of the residual stream that ps_hyper_step takes (csrc/streams.hip)
 
 EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2, "residual": 3, "relu2": 4}
@@ -52,22 +52,23 @@ _SIGNATURES = {
     "ps_softcap": [c_void_p, c_int64, c_int, c_int, c_float, c_void_p],
     "ps_attention_decode": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                            c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
+                            c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int,
                             c_void_p],
     "ps_attention_decode_partial": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                    c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
+                                    c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
     "ps_attention_merge_linear": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                   c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
     "ps_attention_tiled_f32": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                               c_int, c_int, c_int, c_float, c_int, c_void_p],
+                               c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
+                             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
     "ps_attention_mixed": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int,
+                           c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -698,7 +699,7 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
           out.data_ptr(), out_stride, _ptr(partial if splits > 1 else None), floats,
           _ptr(tok_list), _ptr(tok_item), tok_pos.data_ptr(), tables.data_ptr(),
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
-          int(window), int(splits), int(waves), dtype_code(q.dtype), _stream())
+          int(window), int(splits), int(waves), _check_sink(sink, heads), dtype_code(q.dtype), _stream())
     return out
 
 
@@ -740,7 +741,8 @@ def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tabl
     _call("ps_attention_decode_partial", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
           partial.data_ptr(), partial.numel(), _ptr(tok_list), _ptr(tok_item), tok_pos.data_ptr(),
           tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
-          float(scale), int(window), int(splits), int(waves), dtype_code(q.dtype), _stream())
+          float(scale), int(window), int(splits), int(waves), _check_sink(sink, heads),
+          dtype_code(q.dtype), _stream())
     return count
 
 
@@ -857,7 +859,7 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
         step_key = ("prefill", q.data_ptr(), q.shape[0], out.data_ptr(),
                     tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
                     cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale,
-                    window, max_kv_len, query_tile)
+                    window, max_kv_len, query_tile, _ptr(sink))
         key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
         kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
@@ -887,7 +889,7 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
                 out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
                 kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
-                int(query_tile), dtype_code(q.dtype)),
+                int(query_tile), _check_sink(sink, heads), dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 
@@ -937,7 +939,8 @@ def attention_tiled_f32(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, k
     _call("ps_attention_tiled_f32", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
           out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
           cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
-          kv_heads, head_dim, page_size, pages, float(scale), int(window), _stream())
+          kv_heads, head_dim, page_size, pages, float(scale), int(window), _check_sink(sink, heads),
+          _stream())
     return out
 
 
@@ -1004,7 +1007,8 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
         step_key = ("mixed", q.data_ptr(), q.shape[0], out.data_ptr(),
                     tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(), positions.data_ptr(),
                     tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
-                    cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale, window)
+                    cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale, window,
+                    _ptr(sink))
         key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
         kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
@@ -1037,7 +1041,8 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
                 out.data_ptr(), out_stride, tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(),
                 positions.data_ptr(), tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
-                kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype)),
+                kv_heads, head_dim, page_size, pages, float(scale), int(window),
+                _check_sink(sink, heads), dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 

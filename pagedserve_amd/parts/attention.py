@@ -317,10 +317,8 @@ class Attention(Mixer):
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
-                                      tok_list=None if whole else ctx.portion_tokens)
-        kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
-                       packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace),
-                       shared=ctx.shared_calls)
+                                      tok_list=None if whole else ctx.portion_tokens, sink=sink)
+        self._project_out(context, gates, residual, ctx)
 
     def _one_launch(self, singles: int, ctx, tables) -> bool:
         """Whether a step's one-token items and its items of several tokens go to the kernel

@@ -20,7 +20,7 @@ STATIC_ARGS = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_
                c_int, c_int, c_int, c_void_p]
 BUFFER_ARGS = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-               c_int, c_float, c_int, c_int, c_int, c_int, c_void_p]
+               c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
 STATIC_FLOATS = 2 * 1024 * 1024
 
 
@@ -64,9 +64,10 @@ def _both(lib, case, heads, kv_heads, head_dim, page_size, splits, dtype_code):
     q, k_pool, v_pool, tables, tok_item, tok_pos = case
     count = q.shape[0]
     stream = torch.cuda.current_stream().cuda_stream
-    common = (tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], count,
-              heads, kv_heads, head_dim, page_size, k_pool.shape[0], head_dim ** -0.5, 0, splits, 4,
-              dtype_code, stream)
+    sizes = (tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], count,
+             heads, kv_heads, head_dim, page_size, k_pool.shape[0], head_dim ** -0.5, 0, splits, 4)
+    common = sizes + (dtype_code, stream)
+    with_sink = sizes + (None, dtype_code, stream)     # (the buffer variant takes a sink; none here)
     got = torch.full_like(q, float("nan"))
     status = lib.ps_attention_decode_static(q.data_ptr(), q.stride(0), k_pool.data_ptr(),
                                             v_pool.data_ptr(), got.data_ptr(), got.stride(0),
@@ -76,7 +77,7 @@ def _both(lib, case, heads, kv_heads, head_dim, page_size, splits, dtype_code):
     partial = torch.full((count * heads * splits * (head_dim + 2),), float("nan"), device="cuda")
     status = lib.ps_attention_decode(q.data_ptr(), q.stride(0), k_pool.data_ptr(),
                                      v_pool.data_ptr(), expected.data_ptr(), expected.stride(0),
-                                     partial.data_ptr(), partial.numel(), None, *common)
+                                     partial.data_ptr(), partial.numel(), None, *with_sink)
     assert status == 0, lib.ps_last_error().decode()
     torch.cuda.synchronize()
     return got, expected
