@@ -81,6 +81,11 @@ class KosesunConfig:
     max_positions: int
 
     architecture = "Kosesun"
+    eos_token_id = None        # the configuration names no token that ends a request
+
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
     # positions have no bound of their own (rotations): what the cache holds is the limit
     DEFAULT_MAX_POSITIONS = 1 << 20
 

@@ -79,7 +79,9 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
         raise ValueError("max_batch_size must be positive")
     per_page = _bytes_per_page(loaded, block_size, dtype)
     source = "explicit"
-    if num_kv_pages is not None:
+    if per_page == 0:
+        pages = 1        # a model without cached keys (recurrent mixers only): slots are all it holds
+    elif num_kv_pages is not None:
         pages = int(num_kv_pages)
     elif kv_cache_memory_mb is not None:
         if kv_cache_memory_mb <= 0:
