@@ -30,6 +30,7 @@ One JSON line is printed:
     python bench.py --workload medium|small_stream|xl     one workload alone, one JSON line
     python bench.py --prefill-only --steps K [--prefill-length L]   the prefill step of 2 x L tokens alone (for profiles)
     python bench.py --kernels [--shape small|medium|xl|all] [--only name,name]
+    python bench.py --design kosesun [--sizes small,small_narrow,medium]   Kosesun beside GPT-2 at equal size
 
 ``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys), of
 the prefill step (2 x 1,024 tokens) and of a mixed step (32 decoded tokens beside a portion of
@@ -71,7 +72,7 @@ def _random_prompt(generator, length, vocab):
     return torch.randint(0, vocab, (length,), generator=generator).numpy()
 
 
-def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL, pages=None):
+def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL, pages=None, max_context=None):
     """An engine over a model of ``shape`` with random weights (drawn on the GPU: the XL
     shape's 1.5 billion take a second there), and what the weights occupy."""
     import torch
@@ -92,7 +93,7 @@ def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL, pages
     if pages is None:
         pages = max_requests * (config.n_positions // PAGE_SIZE) + 8
     engine = Engine(model, num_pages=pages, page_size=PAGE_SIZE, max_requests=max_requests,
-                    max_step_tokens=max_step_tokens)
+                    max_step_tokens=max_step_tokens, max_context=max_context)
     engine.weights_resident_bytes = resident
     # (as the entry points do once an engine stands: the collector does not walk the model and
     # the modules again in the middle of a timed step)
@@ -494,6 +495,69 @@ def fp32_points(args):
     return points
 
 
+def kosesun_shape(width, layers, heads, kv_heads, dim, vdim, ff, vocab, streams=4, every=4):
+    """A Kosesun configuration of a real model's layer sizes: every ``every``-th layer is gated
+    linear attention, the others attention with grouped heads; all layers mix values."""
+    listed = []
+    for index in range(layers):
+        if index % every == every - 1:
+            mixer = {"heads": heads, "dim": dim, "vdim": dim, "tau": 16.0, "decay_rank": 16}
+            listed.append({"type": "gla", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}})
+        else:
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                     "v_mix": True, "rot": {"dims": dim, "base": 10000.0}}
+            listed.append({"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}})
+    return {"architecture": "Kosesun", "vocab": vocab, "width": width, "streams": streams,
+            "layers": listed, "norm": {"eps": 1e-6}, "embedding": {"scale": width ** 0.5},
+            "logit_softcap": 30.0}
+
+
+# name -> (Kosesun configuration, the GPT-2 shape of equal width, depth, heads, inner width and vocabulary)
+DESIGN_SIZES = {
+    "small": (kosesun_shape(768, 12, 12, 4, 64, 64, 3072, 50257), SMALL),
+    # values half as wide as keys: heads are cached as wide as the keys
+    "small_narrow": (kosesun_shape(768, 12, 12, 4, 64, 32, 3072, 50257), SMALL),
+    "medium": (kosesun_shape(1024, 24, 16, 4, 64, 64, 4096, 50257), MEDIUM),
+}
+
+
+def design_comparison(args):
+    """``--design kosesun``: prefill (2 x 1,024 tokens) and decode (``--batch`` requests whose
+    contexts end at 1,024) throughput of Kosesun models beside GPT-2 models of equal width,
+    depth, head count, inner width and vocabulary, random weights, same engine and scheduler."""
+    import torch
+
+    results = {}
+    context = 1024
+    for name in [piece for piece in args.sizes.split(",") if piece]:
+        if name not in DESIGN_SIZES:
+            raise SystemExit(f"--sizes: unknown size {name!r}; known: {', '.join(DESIGN_SIZES)}")
+        entry = {}
+        for label, raw in zip(("kosesun", "gpt2"), DESIGN_SIZES[name]):
+            pages = 64 * (context // PAGE_SIZE) + 8
+            engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
+                                             shape=raw, pages=pages, max_context=context)
+            seconds = prefill_run(engine, config, reps=8, prompts=2, length=PREFILL_TOKENS // 2)
+            elapsed, _ = decode_run(engine, sampler, config, args.batch, context, args.steps, args.warmup)
+            entry[label] = {
+                "prefill_tokens_per_s": round(PREFILL_TOKENS / seconds, 1),
+                "prefill_ms": round(seconds * 1e3, 3),
+                "decode_tokens_per_s": round(args.batch * args.steps / elapsed, 1),
+                "decode_ms_per_step": round(elapsed / args.steps * 1e3, 4),
+                "parameters": engine.model.parameter_count,
+            }
+            print(f"{name} {label}: {entry[label]}", file=sys.stderr, flush=True)
+            del engine, sampler
+            torch.cuda.empty_cache()
+        entry["prefill_ratio"] = round(entry["kosesun"]["prefill_tokens_per_s"] / entry["gpt2"]["prefill_tokens_per_s"], 3)
+        entry["decode_ratio"] = round(entry["kosesun"]["decode_tokens_per_s"] / entry["gpt2"]["decode_tokens_per_s"], 3)
+        results[name] = entry
+    return {"metric": "prefill tok/s at 2 x 1,024 tokens and decode tok/s, Kosesun beside GPT-2 of equal size",
+            "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "batch": args.batch, "steps": args.steps, "context": context,
+            "data": "synthetic (random weights, uniform-random prompt ids)", "sizes": results}
+
+
 def kernel_tables(args):
     """``--kernels``: the per-kernel tables of ``pagedserve_amd.measure.kernel_table``."""
     from pagedserve_amd.measure import kernel_table as table
@@ -556,6 +620,9 @@ def main(argv=None):
     parser.add_argument("--rows", default="1,8,64", help="decode batch sizes of --kernels")
     parser.add_argument("--only", help="--kernels: only kernels whose name holds one of these (comma-separated)")
     parser.add_argument("--no-prefill", action="store_true", help="--kernels: decode tables only")
+    parser.add_argument("--design", choices=("kosesun",), default=None,
+                        help="prefill and decode throughput of this design beside GPT-2 at equal size")
+    parser.add_argument("--sizes", default="small,small_narrow,medium", help="--design: which sizes")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -566,6 +633,9 @@ def main(argv=None):
     torch.cuda.init()
     if args.kernels:
         print(json.dumps(kernel_tables(args)), flush=True)
+        return 0
+    if args.design:
+        print(json.dumps(design_comparison(args)), flush=True)
         return 0
 
     def rates(default):

@@ -86,8 +86,10 @@ class KosesunConfig:
     @property
     def vocab_size(self) -> int:
         return self.vocab
-    # positions have no bound of their own (rotations): what the cache holds is the limit
-    DEFAULT_MAX_POSITIONS = 1 << 20
+    # positions have no bound of their own (rotations).  Where the file names none, requests may
+    # grow to this many tokens (block tables of 2,048 pages of 16, the widest that the tiled
+    # attention kernel keeps); an engine's pool or its own bound may be smaller.
+    DEFAULT_MAX_POSITIONS = 32768
 
     @classmethod
     def from_dict(cls, raw) -> "KosesunConfig":

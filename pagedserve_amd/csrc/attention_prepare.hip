@@ -32,16 +32,24 @@ __global__ __launch_bounds__(256) void attention_prepare_kernel(
   const float* row = proj + (int64_t)t * ld;
   const int pos = tok_pos[t];
   const int q_cols = heads * key_dim, k_cols = kv_heads * key_dim;
+  // both sums of squares in one pass and one meeting of the block's waves
   float q_inv = 1.f, k_inv = 1.f;
-  if (q_gamma != nullptr) {
-    float sum = 0.f;
-    for (int i = threadIdx.x; i < q_cols; i += blockDim.x) sum = fmaf(row[q_col + i], row[q_col + i], sum);
-    q_inv = 1.0f / sqrtf(block_sum(sum, red) / (float)q_cols + eps);
-  }
-  if (k_gamma != nullptr) {
-    float sum = 0.f;
-    for (int i = threadIdx.x; i < k_cols; i += blockDim.x) sum = fmaf(row[k_col + i], row[k_col + i], sum);
-    k_inv = 1.0f / sqrtf(block_sum(sum, red) / (float)k_cols + eps);
+  if (q_gamma != nullptr || k_gamma != nullptr) {
+    float q_sum = 0.f, k_sum = 0.f;
+    for (int i = threadIdx.x; i < q_cols; i += blockDim.x) q_sum = fmaf(row[q_col + i], row[q_col + i], q_sum);
+    for (int i = threadIdx.x; i < k_cols; i += blockDim.x) k_sum = fmaf(row[k_col + i], row[k_col + i], k_sum);
+    q_sum = wave_sum(q_sum);
+    k_sum = wave_sum(k_sum);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+      red[wave] = q_sum;
+      red[4 + wave] = k_sum;
+    }
+    __syncthreads();
+    q_sum = (red[0] + red[1]) + (red[2] + red[3]);
+    k_sum = (red[4] + red[5]) + (red[6] + red[7]);
+    if (q_gamma != nullptr) q_inv = 1.0f / sqrtf(q_sum / (float)q_cols + eps);
+    if (k_gamma != nullptr) k_inv = 1.0f / sqrtf(k_sum / (float)k_cols + eps);
   }
   const int logical = pos / page_size;
   int page = -1;

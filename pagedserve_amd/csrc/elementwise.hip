@@ -344,16 +344,21 @@ extern "C" int ps_kv_write(const void* k, const void* v, int64_t stride, void* k
   return 0;
 }
 
-// logits <- cap * tanh(logits / cap)
+// logits <- cap * tanh(logits / cap); a row is shared by blocks of 256 columns so that a
+// handful of rows still fills the chip
 __global__ void softcap_kernel(float* __restrict__ logits, int64_t ld, int vocab, float cap) {
-  float* row = logits + (int64_t)blockIdx.x * ld;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) row[i] = cap * tanhf(row[i] / cap);
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i < vocab) {
+    float* p = logits + (int64_t)blockIdx.x * ld + i;
+    *p = cap * tanhf(*p / cap);
+  }
 }
 
 extern "C" int ps_softcap(float* logits, int64_t ld, int rows, int vocab, float cap, void* stream) {
   PS_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab && cap > 0.f, "ps_softcap: bad sizes");
+  PS_REQUIRE((vocab + 255) / 256 <= 65535, "ps_softcap: vocabulary too large");
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(softcap_kernel, dim3(rows), dim3(vocab >= 1024 ? 1024 : 256), 0,
+  hipLaunchKernelGGL(softcap_kernel, dim3(rows, (vocab + 255) / 256), dim3(256), 0,
                      (hipStream_t)stream, logits, ld, vocab, cap);
   PS_CHECK_LAUNCH("ps_softcap");
   return 0;

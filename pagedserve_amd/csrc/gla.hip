@@ -36,14 +36,20 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(
 
 // A block owns GLA_COLS columns of one head's state for one item of the step and walks the
 // item's tokens in order.  The state's rows are dealt to four row groups, RPL rows per lane,
-// in registers; o needs the sum over the row groups (two lane exchanges per token).
+// in registers; o needs the sum over the row groups (two lane exchanges per token).  The
+// tokens' q, k and decays come GLA_CHUNK at a time: a chunk's loads leave together into
+// registers while the chunk before is being worked on from LDS, so that the walk waits for
+// memory once, not once per chunk.
 template <int RPL>
 __global__ __launch_bounds__(64) void gla_scan_kernel(
     const float* __restrict__ proj, int64_t ld, int q_col, int k_col, int v_col,
     const float* __restrict__ alpha, float* __restrict__ state, float* __restrict__ out,
     const int* __restrict__ cu_tokens, const int* __restrict__ slots, int heads, int key_dim,
     int value_dim, float q_scale) {
-  constexpr int PAD = RPL + 4;   // row groups start in different banks
+  constexpr int ROWS = 4 * RPL;                    // rows with padding up to the lanes' share
+  constexpr int PAD = RPL + 4;                     // row groups start in different banks
+  constexpr int PER = GLA_CHUNK * ROWS / 64;       // values of a chunk per lane and array
+  constexpr int PER_V = GLA_CHUNK * GLA_COLS / 64;
   __shared__ float s_q[GLA_CHUNK][4 * PAD];
   __shared__ float s_k[GLA_CHUNK][4 * PAD];
   __shared__ float s_a[GLA_CHUNK][4 * PAD];
@@ -63,31 +69,58 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
     S[i] = (r < key_dim && has_col) ? s_ptr[(int64_t)r * value_dim + col] : 0.f;
   }
   const int channels = heads * key_dim;
-  for (int base = t0; base < t1; base += GLA_CHUNK) {
+  float rq[PER], rk[PER], ra[PER], rv[PER_V];
+  // every load is unconditional from a clamped address; what lies outside is masked when stored
+  auto fetch = [&](const int base) {
     const int count = (t1 - base) < GLA_CHUNK ? (t1 - base) : GLA_CHUNK;
-    __syncthreads();
-    for (int idx = lane; idx < GLA_CHUNK * 4 * RPL; idx += 64) {
-      const int tt = idx / (4 * RPL);
-      const int r = idx - tt * (4 * RPL);
-      const bool valid = tt < count && r < key_dim;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = lane + j * 64;
+      const int tt = idx / ROWS;
+      const int r = idx - tt * ROWS;
       const int64_t t = base + (tt < count ? tt : 0);
       const int c = head * key_dim + (r < key_dim ? r : 0);
-      const float qv = proj[t * ld + q_col + c], kv = proj[t * ld + k_col + c];
-      const float av = alpha[t * channels + c];
-      const int at = (r / RPL) * PAD + (r % RPL);
-      s_q[tt][at] = valid ? qv * q_scale : 0.f;
-      s_k[tt][at] = valid ? kv : 0.f;
-      s_a[tt][at] = valid ? av : 0.f;
+      rq[j] = proj[t * ld + q_col + c];
+      rk[j] = proj[t * ld + k_col + c];
+      ra[j] = alpha[t * channels + c];
     }
-    for (int idx = lane; idx < GLA_CHUNK * GLA_COLS; idx += 64) {
+#pragma unroll
+    for (int j = 0; j < PER_V; ++j) {
+      const int idx = lane + j * 64;
       const int tt = idx / GLA_COLS;
       const int c = blockIdx.z * GLA_COLS + (idx - tt * GLA_COLS);
-      const bool valid = tt < count && c < value_dim;
       const int64_t t = base + (tt < count ? tt : 0);
-      const float vv = proj[t * ld + v_col + head * value_dim + (c < value_dim ? c : 0)];
-      s_v[tt][idx - tt * GLA_COLS] = valid ? vv : 0.f;
+      rv[j] = proj[t * ld + v_col + head * value_dim + (c < value_dim ? c : 0)];
     }
+  };
+  auto stash = [&](const int base) {
+    const int count = (t1 - base) < GLA_CHUNK ? (t1 - base) : GLA_CHUNK;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = lane + j * 64;
+      const int tt = idx / ROWS;
+      const int r = idx - tt * ROWS;
+      const bool valid = tt < count && r < key_dim;
+      const int at = (r / RPL) * PAD + (r % RPL);
+      s_q[tt][at] = valid ? rq[j] * q_scale : 0.f;
+      s_k[tt][at] = valid ? rk[j] : 0.f;
+      s_a[tt][at] = valid ? ra[j] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < PER_V; ++j) {
+      const int idx = lane + j * 64;
+      const int tt = idx / GLA_COLS;
+      const int c = blockIdx.z * GLA_COLS + (idx - tt * GLA_COLS);
+      s_v[tt][idx - tt * GLA_COLS] = (tt < count && c < value_dim) ? rv[j] : 0.f;
+    }
+  };
+  if (t0 < t1) fetch(t0);
+  for (int base = t0; base < t1; base += GLA_CHUNK) {
+    const int count = (t1 - base) < GLA_CHUNK ? (t1 - base) : GLA_CHUNK;
+    __syncthreads();      // the chunk before has been read
+    stash(base);
     __syncthreads();
+    if (base + GLA_CHUNK < t1) fetch(base + GLA_CHUNK);   // in flight during the work below
     for (int tt = 0; tt < count; ++tt) {
       const float v = s_v[tt][lane & 15];
       float o = 0.f;

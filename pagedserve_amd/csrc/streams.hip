@@ -16,73 +16,64 @@
 #define HS_MAX_STREAMS 8
 #define HS_THREADS 256
 
-template <typename TOut, int PER>
+// STREAMS is a template argument so that every loop over the copies is unrolled and a
+// thread's loads of one column (the copies and y) leave together, without a branch between
+// them.  u waits in LDS (width floats) for the row's sum of squares.
+template <typename TOut, int STREAMS>
 __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
     float* __restrict__ X, const float* __restrict__ y, const float* __restrict__ mix,
     const float* __restrict__ out_w, const float* __restrict__ in_w,
     const float* __restrict__ gamma, float eps, TOut* __restrict__ normed,
-    float* __restrict__ zero, int width, int streams) {
+    float* __restrict__ zero, int width) {
+  extern __shared__ float s_u[];
   __shared__ float red[16];
-  __shared__ float s_mix[HS_MAX_STREAMS * HS_MAX_STREAMS];
-  __shared__ float s_out[HS_MAX_STREAMS];
-  __shared__ float s_in[HS_MAX_STREAMS];
   const int t = blockIdx.x;
   const bool writes = y != nullptr;
   const bool reads = normed != nullptr;
-  if (threadIdx.x < streams * streams && writes) s_mix[threadIdx.x] = mix[threadIdx.x];
-  if (threadIdx.x < streams) {
-    if (writes) s_out[threadIdx.x] = out_w[threadIdx.x];
-    if (reads) s_in[threadIdx.x] = in_w[threadIdx.x];
+  // the few weights: every thread reads them itself (the same addresses in all lanes: scalar loads)
+  float w_mix[STREAMS][STREAMS], w_out[STREAMS], w_in[STREAMS];
+#pragma unroll
+  for (int a = 0; a < STREAMS; ++a) {
+    w_out[a] = writes ? out_w[a] : 0.f;
+    w_in[a] = reads ? in_w[a] : 0.f;
+#pragma unroll
+    for (int b = 0; b < STREAMS; ++b) w_mix[a][b] = writes ? mix[a * STREAMS + b] : (a == b ? 1.f : 0.f);
   }
-  __syncthreads();
-  float u[PER];
   float sumsq = 0.f;
-  float* row = X + (int64_t)t * streams * width;
+  float* row = X + (int64_t)t * STREAMS * width;
+  for (int col = threadIdx.x; col < width; col += HS_THREADS) {
+    float x[STREAMS];
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int col = threadIdx.x + i * HS_THREADS;
-    u[i] = 0.f;
-    if (col < width) {
-      float x[HS_MAX_STREAMS];
+    for (int s = 0; s < STREAMS; ++s) x[s] = row[(int64_t)s * width + col];
+    if (writes) {
+      const float yv = y[(int64_t)t * width + col];
+      float nx[STREAMS];
 #pragma unroll
-      for (int s = 0; s < HS_MAX_STREAMS; ++s) x[s] = s < streams ? row[(int64_t)s * width + col] : 0.f;
-      if (writes) {
-        const float yv = y[(int64_t)t * width + col];
-        float nx[HS_MAX_STREAMS];
+      for (int to = 0; to < STREAMS; ++to) {
+        float acc = 0.f;
 #pragma unroll
-        for (int to = 0; to < HS_MAX_STREAMS; ++to) {
-          float acc = 0.f;
-          if (to < streams) {
-#pragma unroll
-            for (int from = 0; from < HS_MAX_STREAMS; ++from)
-              if (from < streams) acc = fmaf(s_mix[from * streams + to], x[from], acc);
-            acc = fmaf(s_out[to], yv, acc);
-            row[(int64_t)to * width + col] = acc;
-          }
-          nx[to] = acc;
-        }
-#pragma unroll
-        for (int s = 0; s < HS_MAX_STREAMS; ++s) x[s] = nx[s];
+        for (int from = 0; from < STREAMS; ++from) acc = fmaf(w_mix[from][to], x[from], acc);
+        nx[to] = fmaf(w_out[to], yv, acc);
+        row[(int64_t)to * width + col] = nx[to];
       }
-      if (reads) {
-        float uu = 0.f;
 #pragma unroll
-        for (int s = 0; s < HS_MAX_STREAMS; ++s)
-          if (s < streams) uu = fmaf(s_in[s], x[s], uu);
-        u[i] = uu;
-        sumsq = fmaf(uu, uu, sumsq);
-      }
-      if (zero != nullptr) zero[(int64_t)t * width + col] = 0.f;
+      for (int s = 0; s < STREAMS; ++s) x[s] = nx[s];
     }
+    if (reads) {
+      float uu = 0.f;
+#pragma unroll
+      for (int s = 0; s < STREAMS; ++s) uu = fmaf(w_in[s], x[s], uu);
+      s_u[col] = uu;
+      sumsq = fmaf(uu, uu, sumsq);
+    }
+    if (zero != nullptr) zero[(int64_t)t * width + col] = 0.f;
   }
   if (!reads) return;
   const float total = block_sum(sumsq, red);
   const float inv = 1.0f / sqrtf(total / (float)width + eps);
-#pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int col = threadIdx.x + i * HS_THREADS;
-    if (col < width) normed[(int64_t)t * width + col] = from_float<TOut>(u[i] * inv * gamma[col]);
-  }
+  // (a thread reads back the columns that it wrote itself)
+  for (int col = threadIdx.x; col < width; col += HS_THREADS)
+    normed[(int64_t)t * width + col] = from_float<TOut>(s_u[col] * inv * gamma[col]);
 }
 
 extern "C" int ps_hyper_step(float* x, const float* y, const float* mix, const float* out_w,
@@ -92,28 +83,33 @@ extern "C" int ps_hyper_step(float* x, const float* y, const float* mix, const f
   PS_REQUIRE(tokens >= 0 && width > 0, "ps_hyper_step: bad sizes");
   PS_REQUIRE(streams >= 1 && streams <= HS_MAX_STREAMS, "ps_hyper_step: %d streams, the kernel takes 1..%d",
              streams, HS_MAX_STREAMS);
-  PS_REQUIRE(width <= HS_THREADS * 32, "ps_hyper_step: width %d above %d", width, HS_THREADS * 32);
+  PS_REQUIRE(width <= 15360, "ps_hyper_step: width %d above 15360 (a row's sums wait in LDS)", width);
   PS_REQUIRE(y == nullptr || (mix != nullptr && out_w != nullptr), "ps_hyper_step: a write needs mix and out weights");
   PS_REQUIRE(normed == nullptr || (in_w != nullptr && gamma != nullptr && eps > 0.f),
              "ps_hyper_step: a read needs in weights, gamma and a positive eps");
   PS_REQUIRE(out_dtype == PS_F32 || out_dtype == PS_BF16, "ps_hyper_step: unknown dtype %d", out_dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-#define PS_LAUNCH_HS(TOut, PER)                                                                  \
-  hipLaunchKernelGGL((hyper_step_kernel<TOut, PER>), dim3(tokens), dim3(HS_THREADS), 0, s, x, y, \
-                     mix, out_w, in_w, gamma, eps, (TOut*)normed, zero, width, streams)
+  const size_t lds = normed != nullptr ? (size_t)width * sizeof(float) : 0;
+#define PS_LAUNCH_HS(TOut, S)                                                                     \
+  hipLaunchKernelGGL((hyper_step_kernel<TOut, S>), dim3(tokens), dim3(HS_THREADS), lds, s, x, y,  \
+                     mix, out_w, in_w, gamma, eps, (TOut*)normed, zero, width)
 #define PS_LAUNCH_HS_T(TOut)                         \
-  do {                                               \
-    const int per = (width + HS_THREADS - 1) / HS_THREADS; \
-    if (per <= 1) PS_LAUNCH_HS(TOut, 1);             \
-    else if (per <= 2) PS_LAUNCH_HS(TOut, 2);        \
-    else if (per <= 4) PS_LAUNCH_HS(TOut, 4);        \
-    else if (per <= 8) PS_LAUNCH_HS(TOut, 8);        \
-    else if (per <= 16) PS_LAUNCH_HS(TOut, 16);      \
-    else PS_LAUNCH_HS(TOut, 32);                     \
-  } while (0)
-  if (out_dtype == PS_F32) PS_LAUNCH_HS_T(float);
-  else PS_LAUNCH_HS_T(bf16_t);
+  switch (streams) {                                 \
+    case 1: PS_LAUNCH_HS(TOut, 1); break;            \
+    case 2: PS_LAUNCH_HS(TOut, 2); break;            \
+    case 3: PS_LAUNCH_HS(TOut, 3); break;            \
+    case 4: PS_LAUNCH_HS(TOut, 4); break;            \
+    case 5: PS_LAUNCH_HS(TOut, 5); break;            \
+    case 6: PS_LAUNCH_HS(TOut, 6); break;            \
+    case 7: PS_LAUNCH_HS(TOut, 7); break;            \
+    default: PS_LAUNCH_HS(TOut, 8); break;           \
+  }
+  if (out_dtype == PS_F32) {
+    PS_LAUNCH_HS_T(float)
+  } else {
+    PS_LAUNCH_HS_T(bf16_t)
+  }
 #undef PS_LAUNCH_HS_T
 #undef PS_LAUNCH_HS
   PS_CHECK_LAUNCH("ps_hyper_step");

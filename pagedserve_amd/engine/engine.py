@@ -75,7 +75,7 @@ class StepError(ValueError):
 
 class Engine:
     def __init__(self, model, num_pages: int, page_size: int = 16, max_requests: int = 64,
-                 max_step_tokens: int = 2048, use_graphs: bool = True):
+                 max_step_tokens: int = 2048, use_graphs: bool = True, max_context: int = None):
         if not torch.cuda.is_available():
             raise RuntimeError("pagedserve_amd runs on a GPU only; no CPU path exists")
         self.model = model
@@ -90,6 +90,11 @@ class Engine:
         # back behind a window) beyond what the pool holds: block tables are that wide.  A model
         # whose positions have no bound of their own (rotations) names a large number.
         self.max_positions = self.spec.max_positions
+        if max_context is not None:
+            # the caller's own bound on a request's length (block tables and launch shapes follow it)
+            if max_context <= 0:
+                raise ValueError("max_context must be positive")
+            self.max_positions = min(self.max_positions, int(max_context))
         if groups and not any(group.window > 0 for group in groups):
             smallest = num_pages if isinstance(num_pages, int) else min(num_pages)
             self.max_positions = min(self.max_positions, smallest * page_size)

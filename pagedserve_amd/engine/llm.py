@@ -41,6 +41,7 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
                     enable_hip_graphs=True, block_size=16, num_kv_pages=None,
                     max_num_batched_tokens=None, max_prefill_requests=None, random_weights=False,
                     seed=0, eos_token_id="config", model_name=None, enable_cuda_graphs=None,
+                    max_model_len=None,
                     decode_attention_backend="hip", kv_cache_dtype="model"):
     """Load ``model`` (a folder, or a preset's name such as ``"reference"`` for a small random
     model) and return a ``ContinuousBatchScheduler`` ready for ``add_request`` /
@@ -93,14 +94,15 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
         budget = kv_cache_budget(free_memory, total_memory, kv_cache_memory_utilization,
                                  kv_cache_safety_mb * MIB)
         # never more than every slot at full context needs
-        useful = max_batch_size * (-(-loaded.spec.max_positions // block_size)) * per_page
+        longest = min(loaded.spec.max_positions, max_model_len or loaded.spec.max_positions)
+        useful = max_batch_size * (-(-longest // block_size)) * per_page
         pages = min(budget, useful) // per_page
         source = "device_auto"
     if pages <= 0:
         raise ValueError(f"Memory budget is too small; one block requires {per_page} bytes")
     step_tokens = max_num_batched_tokens or max(2048, max_batch_size)
     engine = Engine(loaded, num_pages=pages, page_size=block_size, max_requests=max_batch_size,
-                    max_step_tokens=step_tokens, use_graphs=enable_hip_graphs)
+                    max_step_tokens=step_tokens, use_graphs=enable_hip_graphs, max_context=max_model_len)
     engine.memory_budget_source = source
     from ..sampling.sampler import Sampler
 
