@@ -31,33 +31,37 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(
   }
 }
 
-#define GLA_COLS 16    // value columns per block (one wave): lane = row group * 16 + column
-#define GLA_CHUNK 8    // tokens whose q, k, alpha are staged in LDS at a time
 
-// A block owns GLA_COLS columns of one head's state for one item of the step and walks the
-// item's tokens in order.  The state's rows are dealt to four row groups, RPL rows per lane,
-// in registers; o needs the sum over the row groups (two lane exchanges per token).  The
-// tokens' q, k and decays come GLA_CHUNK at a time: a chunk's loads leave together into
-// registers while the chunk before is being worked on from LDS, so that the walk waits for
-// memory once, not once per chunk.
-template <int RPL>
+// A block (one wave) owns COLS columns of one head's state for one item of the step and walks
+// the item's tokens in order: lane = row group * COLS + column.  The state's rows are dealt to
+// the 64 / COLS row groups, RPL rows per lane, in registers; o needs the sum over the row groups
+// (lane exchanges per token).  The walk is one dependent chain per token, so a launch with few
+// blocks takes narrow ones (4 columns, 16 row groups: a quarter of the work per lane and token,
+// four times the blocks), one with many the wide ones (16 columns, 4 row groups).  The
+// tokens' q, k and decays come GLA_CHUNK at a time (32 for key heads up to 64, fewer for larger
+// ones: 32 values per lane and array): a chunk's loads leave together into registers while the
+// chunk before is being worked on from LDS; the work on a chunk has to last as long as a trip
+// to memory for the walk not to wait, hence chunks as long as the registers allow.
+template <int RPL, int COLS, int GLA_CHUNK>
 __global__ __launch_bounds__(64) void gla_scan_kernel(
     const float* __restrict__ proj, int64_t ld, int q_col, int k_col, int v_col,
     const float* __restrict__ alpha, float* __restrict__ state, float* __restrict__ out,
     const int* __restrict__ cu_tokens, const int* __restrict__ slots, int heads, int key_dim,
     int value_dim, float q_scale) {
-  constexpr int ROWS = 4 * RPL;                    // rows with padding up to the lanes' share
+  constexpr int GROUPS = 64 / COLS;                // row groups
+  constexpr int ROWS = GROUPS * RPL;               // rows with padding up to the lanes' share
   constexpr int PAD = RPL + 4;                     // row groups start in different banks
   constexpr int PER = GLA_CHUNK * ROWS / 64;       // values of a chunk per lane and array
-  constexpr int PER_V = GLA_CHUNK * GLA_COLS / 64;
-  __shared__ float s_q[GLA_CHUNK][4 * PAD];
-  __shared__ float s_k[GLA_CHUNK][4 * PAD];
-  __shared__ float s_a[GLA_CHUNK][4 * PAD];
-  __shared__ float s_v[GLA_CHUNK][GLA_COLS];
+  constexpr int PER_V = (GLA_CHUNK * COLS + 63) / 64;
+  static_assert(GLA_CHUNK * ROWS % 64 == 0 && PER >= 1, "a chunk's rows are dealt evenly to the lanes");
+  __shared__ __attribute__((aligned(16))) float s_q[GLA_CHUNK][GROUPS * PAD];
+  __shared__ __attribute__((aligned(16))) float s_k[GLA_CHUNK][GROUPS * PAD];
+  __shared__ __attribute__((aligned(16))) float s_a[GLA_CHUNK][GROUPS * PAD];
+  __shared__ float s_v[GLA_CHUNK][COLS];
   const int item = blockIdx.x, head = blockIdx.y;
   const int lane = threadIdx.x;
-  const int col = blockIdx.z * GLA_COLS + (lane & 15);
-  const int group = lane >> 4;
+  const int col = blockIdx.z * COLS + (lane % COLS);
+  const int group = lane / COLS;
   const bool has_col = col < value_dim;
   const int t0 = cu_tokens[item], t1 = cu_tokens[item + 1];
   const int slot = slots[item];
@@ -86,9 +90,9 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
     }
 #pragma unroll
     for (int j = 0; j < PER_V; ++j) {
-      const int idx = lane + j * 64;
-      const int tt = idx / GLA_COLS;
-      const int c = blockIdx.z * GLA_COLS + (idx - tt * GLA_COLS);
+      const int idx = (lane + j * 64) % (GLA_CHUNK * COLS);
+      const int tt = idx / COLS;
+      const int c = blockIdx.z * COLS + (idx - tt * COLS);
       const int64_t t = base + (tt < count ? tt : 0);
       rv[j] = proj[t * ld + v_col + head * value_dim + (c < value_dim ? c : 0)];
     }
@@ -109,9 +113,11 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
 #pragma unroll
     for (int j = 0; j < PER_V; ++j) {
       const int idx = lane + j * 64;
-      const int tt = idx / GLA_COLS;
-      const int c = blockIdx.z * GLA_COLS + (idx - tt * GLA_COLS);
-      s_v[tt][idx - tt * GLA_COLS] = (tt < count && c < value_dim) ? rv[j] : 0.f;
+      if (idx < GLA_CHUNK * COLS) {
+        const int tt = idx / COLS;
+        const int c = blockIdx.z * COLS + (idx - tt * COLS);
+        s_v[tt][idx - tt * COLS] = (tt < count && c < value_dim) ? rv[j] : 0.f;
+      }
     }
   };
   if (t0 < t1) fetch(t0);
@@ -121,8 +127,9 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
     stash(base);
     __syncthreads();
     if (base + GLA_CHUNK < t1) fetch(base + GLA_CHUNK);   // in flight during the work below
-    for (int tt = 0; tt < count; ++tt) {
-      const float v = s_v[tt][lane & 15];
+    // a lane's share of o_t
+    auto token = [&](const int tt) -> float {
+      const float v = s_v[tt][lane % COLS];
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < RPL; ++i) {
@@ -130,10 +137,24 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
         S[i] = fmaf(s_a[tt][at], S[i], s_k[tt][at] * v);
         o = fmaf(S[i], s_q[tt][at], o);
       }
+      return o;
+    };
+    // over the lanes with the same column: rotations inside the row of 16 lanes, then the
+    // swaps of rows and halves
+    auto finish = [&](float o, const int tt) {
+      if (COLS <= 4) o += lane_exchange<0x124>(o);     // row_ror:4
+      if (COLS <= 8) o += lane_exchange<0x128>(o);     // row_ror:8
       o = xor_sum<16>(o);
       o = xor_sum<32>(o);
       if (group == 0 && has_col)
         out[(int64_t)(base + tt) * heads * value_dim + head * value_dim + col] = o;
+    };
+    if (count == GLA_CHUNK) {
+      // a whole chunk: unrolled, so that the reads and sums of neighbouring tokens overlap
+#pragma unroll
+      for (int tt = 0; tt < GLA_CHUNK; ++tt) finish(token(tt), tt);
+    } else {
+      for (int tt = 0; tt < count; ++tt) finish(token(tt), tt);
     }
   }
 #pragma unroll
@@ -183,22 +204,44 @@ extern "C" int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank
 extern "C" int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
                            const float* alpha, float* state, float* out, const int* cu_tokens,
                            const int* slots, int items, int max_slots, int heads, int key_dim,
-                           int value_dim, float q_scale, void* stream) {
+                           int value_dim, float q_scale, int longest, void* stream) {
   PS_REQUIRE(items >= 0 && heads > 0 && key_dim > 0 && value_dim > 0 && max_slots > 0,
              "ps_gla_scan: bad sizes");
   PS_REQUIRE(key_dim <= 256, "ps_gla_scan: key head size %d above 256", key_dim);
-  PS_REQUIRE(heads <= 65535 && (value_dim + GLA_COLS - 1) / GLA_COLS <= 65535, "ps_gla_scan: grid too large");
+  PS_REQUIRE(heads <= 65535 && (value_dim + 3) / 4 <= 65535, "ps_gla_scan: grid too large");
   if (items == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid(items, heads, (value_dim + GLA_COLS - 1) / GLA_COLS);
-#define PS_LAUNCH_GLA(RPL)                                                                       \
-  hipLaunchKernelGGL((gla_scan_kernel<RPL>), grid, dim3(64), 0, s, proj, ld, q_col, k_col, v_col, \
-                     alpha, state, out, cu_tokens, slots, heads, key_dim, value_dim, q_scale)
-  if (key_dim <= 32) PS_LAUNCH_GLA(8);
-  else if (key_dim <= 64) PS_LAUNCH_GLA(16);
-  else if (key_dim <= 128) PS_LAUNCH_GLA(32);
-  else PS_LAUNCH_GLA(64);
+  // narrow blocks while wide ones would leave the chip's SIMDs (four to a compute unit) idle
+  const int64_t wide_blocks = (int64_t)items * heads * ((value_dim + 15) / 16);
+  const bool narrow = wide_blocks < 2 * (int64_t)ps_compute_units();
+  // items of a few tokens at most (decode steps): chunks of 8, which cost less to stage
+  const bool brief = longest > 0 && longest <= 8;
+#define PS_LAUNCH_GLA_C(RPL, COLS, CHUNK)                                                         \
+  hipLaunchKernelGGL((gla_scan_kernel<RPL, COLS, CHUNK>),                                         \
+                     dim3(items, heads, (value_dim + COLS - 1) / COLS),                           \
+                     dim3(64), 0, s, proj, ld, q_col, k_col, v_col, alpha, state, out, cu_tokens, \
+                     slots, heads, key_dim, value_dim, q_scale)
+#define PS_LAUNCH_GLA(RPL, COLS)                                                                  \
+  do {                                                                                            \
+    if (brief) {                                                                                  \
+      PS_LAUNCH_GLA_C(RPL, COLS, 8);                                                              \
+    } else {                                                                                      \
+      PS_LAUNCH_GLA_C(RPL, COLS, (2048 / (64 / COLS * RPL) < 32 ? 2048 / (64 / COLS * RPL) : 32)); \
+    }                                                                                             \
+  } while (0)
+  if (narrow) {
+    if (key_dim <= 32) PS_LAUNCH_GLA(2, 4);
+    else if (key_dim <= 64) PS_LAUNCH_GLA(4, 4);
+    else if (key_dim <= 128) PS_LAUNCH_GLA(8, 4);
+    else PS_LAUNCH_GLA(16, 4);
+  } else {
+    if (key_dim <= 32) PS_LAUNCH_GLA(8, 16);
+    else if (key_dim <= 64) PS_LAUNCH_GLA(16, 16);
+    else if (key_dim <= 128) PS_LAUNCH_GLA(32, 16);
+    else PS_LAUNCH_GLA(64, 16);
+  }
 #undef PS_LAUNCH_GLA
+#undef PS_LAUNCH_GLA_C
   PS_CHECK_LAUNCH("ps_gla_scan");
   return 0;
 }

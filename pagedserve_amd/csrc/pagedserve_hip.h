@@ -281,11 +281,12 @@ int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank, const voi
 // For every item i of the step (tokens cu_tokens[i] .. cu_tokens[i + 1] - 1, state slot
 // slots[i]) and head: S = diag(alpha_t) S + k_t v_t^T, out[t] = S^T (q_t * q_scale), token after
 // token; state: [max_slots, heads, key_dim, value_dim] float, read at the start and written
-// back at the end; out: [tokens, heads * value_dim] float.
+// back at the end; out: [tokens, heads * value_dim] float.  longest: no item brings more
+// tokens than that (0: unknown); it only steers the launch shape.
 int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
                 const float* alpha, float* state, float* out, const int* cu_tokens,
                 const int* slots, int items, int max_slots, int heads, int key_dim, int value_dim,
-                float q_scale, void* stream);
+                float q_scale, int longest, void* stream);
 // out[t, h, :] = rms_norm(o[t, h, :]) * w * silu(gate[t * gate_ld + h * value_dim ...]).
 int ps_gla_output(const float* o, const float* w, float eps, const float* gate, int64_t gate_ld,
                   void* out, int64_t out_stride, int tokens, int heads, int value_dim, int dtype,

@@ -46,7 +46,7 @@ _SIGNATURES = {
     "ps_gla_decay": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int,
                      c_int, c_int, c_void_p],
     "ps_gla_scan": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "ps_gla_output": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
                       c_int, c_int, c_int, c_void_p],
     "ps_softcap": [c_void_p, c_int64, c_int, c_int, c_float, c_void_p],
@@ -1177,9 +1177,11 @@ def gla_decay(proj, low_col, w, bias, tau, alpha):
           float(tau), alpha.data_ptr(), tokens, channels, dtype_code(w.dtype), _stream())
 
 
-def gla_scan(proj, columns, alpha, state, out, cu_tokens, slots, heads, key_dim, value_dim, q_scale):
+def gla_scan(proj, columns, alpha, state, out, cu_tokens, slots, heads, key_dim, value_dim, q_scale,
+             longest=0):
     """The recurrence of gated linear attention over the step's items, token after token
-    (``csrc/pagedserve_hip.h: ps_gla_scan``); ``state``: float ``[slots, heads, key_dim, value_dim]``."""
+    (``csrc/pagedserve_hip.h: ps_gla_scan``); ``state``: float ``[slots, heads, key_dim, value_dim]``.
+    ``longest``: no item brings more tokens than that (0: unknown); it steers the launch shape only."""
     _check(proj, "proj", torch.float32, 2)
     tokens = proj.shape[0]
     q_col, k_col, v_col = columns
@@ -1197,7 +1199,7 @@ def gla_scan(proj, columns, alpha, state, out, cu_tokens, slots, heads, key_dim,
         raise KernelError("gla_scan: cu_tokens must hold one entry more than slots")
     _call("ps_gla_scan", proj.data_ptr(), _rows(proj, "proj"), q_col, k_col, v_col, alpha.data_ptr(),
           state.data_ptr(), out.data_ptr(), cu_tokens.data_ptr(), slots.data_ptr(), items,
-          state.shape[0], heads, key_dim, value_dim, float(q_scale), _stream())
+          state.shape[0], heads, key_dim, value_dim, float(q_scale), int(longest), _stream())
 
 
 def gla_output(o, weight, eps, gate, out, heads, value_dim):

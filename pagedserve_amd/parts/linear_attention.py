@@ -87,7 +87,8 @@ class GatedLinearAttention(Mixer):
         kernels.gla_decay(proj, low_col, self.decay_weight, self.decay_bias, self.tau, alpha)
         raw = workspace.first_rows("gla_raw", self.v_cols, torch.float32, tokens)
         kernels.gla_scan(proj, (q_col, k_col, v_col), alpha, cache.state, raw, ctx.cu_tokens,
-                         ctx.slots, self.heads, self.key_dim, self.value_dim, self.key_dim ** -0.5)
+                         ctx.slots, self.heads, self.key_dim, self.value_dim, self.key_dim ** -0.5,
+                         longest=1 if ctx.decode_only else 0)
         gated = workspace.first_rows("gla_out", self.v_cols, self.dtype, tokens)
         kernels.gla_output(raw, self.norm_gamma, self.norm_eps, proj[:, gate_col:gate_col + self.v_cols],
                            gated, self.heads, self.value_dim)

@@ -322,11 +322,11 @@ def test_decay_is_right_at_both_ends():
 @pytest.mark.parametrize("heads,dim,vdim", [(2, 16, 24), (1, 40, 72), (3, 8, 8), (2, 64, 64), (1, 130, 20)])
 def test_recurrence_in_one_go_in_pieces_and_in_reused_slots(heads, dim, vdim):
     """Several requests of unequal length in one launch against the plain recurrence; the same
-    tokens cut into pieces (1, 7, 8 and 9 tokens: the kernel stages 8 at a time) give the same
+    tokens cut into pieces (around the 8 and the 32 tokens that the kernel stages at a time) give the same
     state and outputs; a slot that is cleared and used again carries nothing over."""
     kernels = _kernels()
     g = torch.Generator().manual_seed(heads * 100 + dim)
-    lengths = [25, 1, 9]
+    lengths = [107, 1, 9]
     slots = [2, 0, 3]
     total = sum(lengths)
     q_col, k_col, v_col = 2, 2 + heads * dim, 2 + 2 * heads * dim
@@ -358,17 +358,52 @@ def test_recurrence_in_one_go_in_pieces_and_in_reused_slots(heads, dim, vdim):
     state[0].zero_()
     cursor = 0
     pieces = []
-    for size in (1, 7, 8, 9):
+    for size, longest in ((1, 1), (7, 0), (8, 8), (9, 0), (33, 0), (32, 0), (17, 0)):
         rows = slice(cursor, cursor + size)
         piece = torch.empty((size, heads * vdim), device="cuda")
         kernels.gla_scan(proj[rows].cuda(), (q_col, k_col, v_col), alpha[rows].cuda(), state, piece,
                          torch.tensor([0, size], dtype=torch.int32, device="cuda"),
-                         torch.tensor([0], dtype=torch.int32, device="cuda"), heads, dim, vdim, scale)
+                         torch.tensor([0], dtype=torch.int32, device="cuda"), heads, dim, vdim, scale,
+                         longest=longest)
         pieces.append(piece)
         cursor += size
     assert cursor == lengths[0]
     assert torch.allclose(torch.cat(pieces), out[:cursor], atol=1e-5, rtol=1e-5)
     assert torch.allclose(state[0].double().cpu(), finals[0], atol=2e-4, rtol=2e-4)
+
+
+@pytest.mark.parametrize("heads,dim,vdim", [(3, 24, 64), (2, 100, 144)])
+def test_recurrence_of_many_requests_at_once(heads, dim, vdim):
+    """So many (request, head, column block) triples that the kernel takes its wide blocks."""
+    kernels = _kernels()
+    g = torch.Generator().manual_seed(dim)
+    count = 2 * kernels.compute_units() // (heads * -(-vdim // 16)) + 1
+    lengths = [1 + (n * 5) % 11 for n in range(count)]
+    total = sum(lengths)
+    q_col, k_col, v_col = 0, heads * dim, 2 * heads * dim
+    proj = torch.randn((total, v_col + heads * vdim), generator=g)
+    alpha = torch.rand((total, heads * dim), generator=g) * 0.6 + 0.4
+    initial = torch.randn((count + 1, heads, dim, vdim), generator=g)
+    state = initial.clone().cuda()
+    slots = torch.randperm(count, generator=g).tolist()
+    out = torch.full((total, heads * vdim), float("nan"), device="cuda")
+    cu = [0]
+    for length in lengths:
+        cu.append(cu[-1] + length)
+    kernels.gla_scan(proj.cuda(), (q_col, k_col, v_col), alpha.cuda(), state, out,
+                     torch.tensor(cu, dtype=torch.int32, device="cuda"),
+                     torch.tensor(slots, dtype=torch.int32, device="cuda"), heads, dim, vdim, 0.5)
+    got, final = out.double().cpu(), state.double().cpu()
+    for n in range(0, count, 7):
+        rows, length = slice(cu[n], cu[n + 1]), lengths[n]
+        o, last = plain.gated_recurrence(
+            proj[rows, :k_col].double().view(length, heads, dim) * 0.5,
+            proj[rows, k_col:v_col].double().view(length, heads, dim),
+            proj[rows, v_col:].double().view(length, heads, vdim),
+            alpha[rows].double().view(length, heads, dim), initial[slots[n]].double())
+        assert torch.allclose(got[rows].view(length, heads, vdim), o, atol=5e-4, rtol=5e-4)
+        assert torch.allclose(final[slots[n]], last, atol=5e-4, rtol=5e-4)
+    assert torch.equal(final[count].float(), initial[count])
 
 
 def test_recurrent_output_norm_and_gate():
