@@ -19,7 +19,7 @@
 #include "pagedserve_hip.h"
 
 template <typename T>
-__global__ __launch_bounds__(256) void attention_prepare_kernel(
+__global__ __launch_bounds__(1024) void attention_prepare_kernel(
     const float* __restrict__ proj, int64_t ld, int q_col, int k_col, int v_col,
     T* __restrict__ q_out, int64_t q_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
     const float* __restrict__ q_gamma, const float* __restrict__ k_gamma, float eps,
@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void attention_prepare_kernel(
     const float* __restrict__ v_lambda, int v_mode, const int* __restrict__ tok_item,
     const int* __restrict__ tok_pos, const int* __restrict__ tables, int table_width, int heads,
     int kv_heads, int key_dim, int value_dim, int cache_dim, int page_size, int num_pages) {
-  __shared__ float red[16];
+  __shared__ float red[2][16];
   const int t = blockIdx.x;
   const float* row = proj + (int64_t)t * ld;
   const int pos = tok_pos[t];
@@ -41,13 +41,18 @@ __global__ __launch_bounds__(256) void attention_prepare_kernel(
     q_sum = wave_sum(q_sum);
     k_sum = wave_sum(k_sum);
     const int wave = threadIdx.x >> 6;
+    const int waves = (blockDim.x + 63) >> 6;
     if ((threadIdx.x & 63) == 0) {
-      red[wave] = q_sum;
-      red[4 + wave] = k_sum;
+      red[0][wave] = q_sum;
+      red[1][wave] = k_sum;
     }
     __syncthreads();
-    q_sum = (red[0] + red[1]) + (red[2] + red[3]);
-    k_sum = (red[4] + red[5]) + (red[6] + red[7]);
+    q_sum = 0.f;
+    k_sum = 0.f;
+    for (int w = 0; w < waves; ++w) {
+      q_sum += red[0][w];
+      k_sum += red[1][w];
+    }
     if (q_gamma != nullptr) q_inv = 1.0f / sqrtf(q_sum / (float)q_cols + eps);
     if (k_gamma != nullptr) k_inv = 1.0f / sqrtf(k_sum / (float)k_cols + eps);
   }
@@ -131,14 +136,20 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_prepare: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  // as many threads as the widest of the three passes has elements (the queries' columns, the
+  // pairs of queries and keys), so that a pass is one round of loads where the row allows
+  int widest = heads * key_dim;
+  if ((heads + kv_heads) * (cache_dim / 2) > widest) widest = (heads + kv_heads) * (cache_dim / 2);
+  int threads = widest >= 1024 ? 1024 : (widest + 63) / 64 * 64;
+  if (tokens > 256 && threads > 256) threads = 256;   // (many rows fill the chip anyway)
   if (dtype == PS_F32)
-    hipLaunchKernelGGL(attention_prepare_kernel<float>, dim3(tokens), dim3(256), 0, s, proj, ld, q_col,
+    hipLaunchKernelGGL(attention_prepare_kernel<float>, dim3(tokens), dim3(threads), 0, s, proj, ld, q_col,
                        k_col, v_col, (float*)q_out, q_stride, (float*)k_pool, (float*)v_pool, q_gamma,
                        k_gamma, eps, freqs, rot_dims, (float*)v_first, v_lambda, v_mode, tok_item,
                        tok_pos, tables, table_width, heads, kv_heads, key_dim, value_dim, cache_dim,
                        page_size, num_pages);
   else
-    hipLaunchKernelGGL(attention_prepare_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, proj, ld, q_col,
+    hipLaunchKernelGGL(attention_prepare_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s, proj, ld, q_col,
                        k_col, v_col, (bf16_t*)q_out, q_stride, (bf16_t*)k_pool, (bf16_t*)v_pool,
                        q_gamma, k_gamma, eps, freqs, rot_dims, (bf16_t*)v_first, v_lambda, v_mode,
                        tok_item, tok_pos, tables, table_width, heads, kv_heads, key_dim, value_dim,

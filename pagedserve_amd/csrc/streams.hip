@@ -14,7 +14,8 @@
 #include "pagedserve_hip.h"
 
 #define HS_MAX_STREAMS 8
-#define HS_THREADS 256
+#define HS_THREADS 1024   // at most; a launch takes as many as the row has columns, so that a
+                          // row of up to 1,024 columns is one round of loads
 
 // STREAMS is a template argument so that every loop over the copies is unrolled and a
 // thread's loads of one column (the copies and y) leave together, without a branch between
@@ -41,7 +42,7 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
   }
   float sumsq = 0.f;
   float* row = X + (int64_t)t * STREAMS * width;
-  for (int col = threadIdx.x; col < width; col += HS_THREADS) {
+  for (int col = threadIdx.x; col < width; col += blockDim.x) {
     float x[STREAMS];
 #pragma unroll
     for (int s = 0; s < STREAMS; ++s) x[s] = row[(int64_t)s * width + col];
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
   const float total = block_sum(sumsq, red);
   const float inv = 1.0f / sqrtf(total / (float)width + eps);
   // (a thread reads back the columns that it wrote itself)
-  for (int col = threadIdx.x; col < width; col += HS_THREADS)
+  for (int col = threadIdx.x; col < width; col += blockDim.x)
     normed[(int64_t)t * width + col] = from_float<TOut>(s_u[col] * inv * gamma[col]);
 }
 
@@ -91,8 +92,12 @@ extern "C" int ps_hyper_step(float* x, const float* y, const float* mix, const f
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const size_t lds = normed != nullptr ? (size_t)width * sizeof(float) : 0;
+  // few rows wait for their trips to memory: a thread per column; many rows fill the chip
+  // anyway and run faster as blocks of four waves that walk their row
+  int threads = width >= HS_THREADS ? HS_THREADS : (width + 63) / 64 * 64;
+  if (tokens > 256 && threads > 256) threads = 256;
 #define PS_LAUNCH_HS(TOut, S)                                                                     \
-  hipLaunchKernelGGL((hyper_step_kernel<TOut, S>), dim3(tokens), dim3(HS_THREADS), lds, s, x, y,  \
+  hipLaunchKernelGGL((hyper_step_kernel<TOut, S>), dim3(tokens), dim3(threads), lds, s, x, y,     \
                      mix, out_w, in_w, gamma, eps, (TOut*)normed, zero, width)
 #define PS_LAUNCH_HS_T(TOut)                         \
   switch (streams) {                                 \
