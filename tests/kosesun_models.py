@@ -54,8 +54,22 @@ MODEL_D = {
                _gla(2, 64, 64, 16.0, 256),
                _attention(4, 2, 64, 64, 32, 10000.0, 0.125, True, 256)],
 }
+# recurrent layers only (nothing is paged), two copies, one layer without a feed-forward
+MODEL_E = {
+    "architecture": "Kosesun", "vocab": 77, "width": 40, "streams": 2,
+    "norm": {"eps": 1e-5}, "embedding": {"scale": 3.0},
+    "layers": [_gla(2, 12, 20, 4.0, 56), _gla(5, 4, 4, 64.0, None), _gla(2, 12, 20, 4.0, 56)],
+}
+# attention only, sizes that are multiples of nothing (width 100, five heads of 12, a vocabulary of
+# 51), eight copies, a single layer
+MODEL_F = {
+    "architecture": "Kosesun", "vocab": 51, "width": 100, "streams": 8, "logit_softcap": 5.0,
+    "norm": {"eps": 1e-6}, "embedding": {"scale": 10.0},
+    "layers": [_attention(5, 5, 12, 12, 6, 100.0, 0.4, True, 36)],
+}
 # name -> (configuration, page size, seed, rank of the decay projection)
-MODELS = {"A": (MODEL_A, 8, 0, 4), "B": (MODEL_B, 16, 1, 3), "C": (MODEL_C, 4, 2, 6), "D": (MODEL_D, 16, 3, 16)}
+MODELS = {"A": (MODEL_A, 8, 0, 4), "B": (MODEL_B, 16, 1, 3), "C": (MODEL_C, 4, 2, 6), "D": (MODEL_D, 16, 3, 16),
+          "E": (MODEL_E, 8, 4, 2), "F": (MODEL_F, 16, 5, 1)}
 
 
 def folder_of(tmp_path, which):

@@ -72,6 +72,9 @@ def test_every_parameter_has_a_source_and_every_tensor_a_parameter(tmp_path):
         # the one stored tensor that nothing reads: the mixing weight of the source layer
         assert len(unused) == (1 if any(l["type"] == "attention" and l["mixer"]["v_mix"]
                                         for l in raw["layers"]) else 0)
+        groups, states = model.cache_requirements()
+        assert len(states) == sum(l["type"] == "gla" for l in raw["layers"])
+        assert bool(groups) == any(l["type"] == "attention" for l in raw["layers"])
         # the decay rank came from the tensor's shape
         for index, layer in enumerate(raw["layers"]):
             if layer["type"] == "gla":
