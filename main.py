@@ -57,6 +57,9 @@ def parse_args(argv=None):
     parser.add_argument("--prompt", action="append", help="text prompt (may be repeated)")
     parser.add_argument("--prompt-ids", action="append",
                         help="prompt as comma- or space-separated token ids (may be repeated)")
+    parser.add_argument("--max-model-len", type=int,
+                        help="longest request (prompt and output) that the engine takes; for models whose "
+                             "positions have no bound of their own")
     parser.add_argument("--max-new-tokens", type=int, default=8)
     parser.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
     parser.add_argument("--sample-seed", type=int, help="seed of temperature sampling")
@@ -79,7 +82,7 @@ def main(argv=None):
         kv_cache_safety_mb=args.kv_cache_safety_mb, execution_dtype=args.dtype,
         enable_hip_graphs=not args.disable_hip_graphs, block_size=args.block_size,
         num_kv_pages=args.num_kv_pages, max_num_batched_tokens=args.max_num_batched_tokens,
-        random_weights=args.random_weights, seed=args.seed)
+        random_weights=args.random_weights, seed=args.seed, max_model_len=args.max_model_len)
     sampling = SamplingParams(temperature=args.temperature, seed=args.sample_seed,
                               max_new_tokens=args.max_new_tokens, ignore_eos=args.ignore_eos)
     request_ids = []
