@@ -32,12 +32,55 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
   const float* row = proj + (int64_t)t * ld;
   const int pos = tok_pos[t];
   const int q_cols = heads * key_dim, k_cols = kv_heads * key_dim;
-  // both sums of squares in one pass and one meeting of the block's waves
+  const int logical = pos / page_size;
+  int page = -1;
+  if (logical < table_width) page = tables[(int64_t)tok_item[t] * table_width + logical];
+  const bool stored = page >= 0 && page < num_pages;
+  const int offset = pos - logical * page_size;
+  const int half = cache_dim / 2;   // cache_dim is even
+  // Queries and keys, a pair of neighbouring dimensions per thread and turn.  A pair's values,
+  // weights and rotation do not wait for the norms: a thread loads and turns its first pair
+  // before the block meets for the sums of squares (which the same values feed), so that a
+  // step of few tokens makes one trip to memory; further pairs of a thread are read again.
+  const int q_pairs = heads * half, k_pairs = kv_heads * half;
+  struct Pair {
+    float a, b, wa, wb, cs, sn;
+    int head, d0;
+    bool is_q;
+  };
+  auto load_pair = [&](const int i) -> Pair {
+    Pair p;
+    p.is_q = i < q_pairs;
+    const int j = p.is_q ? i : i - q_pairs;
+    p.head = j / half;
+    p.d0 = (j - p.head * half) * 2;
+    const int src = (p.is_q ? q_col : k_col) + p.head * key_dim + p.d0;
+    const float* gamma = p.is_q ? q_gamma : k_gamma;
+    p.a = p.d0 < key_dim ? row[src] : 0.f;
+    p.b = p.d0 + 1 < key_dim ? row[src + 1] : 0.f;
+    p.wa = (gamma && p.d0 < key_dim) ? gamma[p.head * key_dim + p.d0] : 1.f;
+    p.wb = (gamma && p.d0 + 1 < key_dim) ? gamma[p.head * key_dim + p.d0 + 1] : 1.f;
+    p.cs = 1.f;
+    p.sn = 0.f;
+    if (p.d0 + 1 < rot_dims) sincosf((float)pos * freqs[p.d0 >> 1], &p.sn, &p.cs);
+    return p;
+  };
+  const int pairs = q_pairs + k_pairs;
+  const bool has_first = (int)threadIdx.x < pairs;
+  Pair first = {};
+  if (has_first) first = load_pair(threadIdx.x);
   float q_inv = 1.f, k_inv = 1.f;
   if (q_gamma != nullptr || k_gamma != nullptr) {
     float q_sum = 0.f, k_sum = 0.f;
-    for (int i = threadIdx.x; i < q_cols; i += blockDim.x) q_sum = fmaf(row[q_col + i], row[q_col + i], q_sum);
-    for (int i = threadIdx.x; i < k_cols; i += blockDim.x) k_sum = fmaf(row[k_col + i], row[k_col + i], k_sum);
+    if (has_first) {
+      const float sq = first.a * first.a + first.b * first.b;
+      if (first.is_q) q_sum = sq; else k_sum = sq;
+    }
+    for (int i = threadIdx.x + blockDim.x; i < pairs; i += blockDim.x) {
+      const Pair p = load_pair(i);
+      const float sq = p.a * p.a + p.b * p.b;
+      if (p.is_q) q_sum += sq; else k_sum += sq;
+    }
     q_sum = wave_sum(q_sum);
     k_sum = wave_sum(k_sum);
     const int wave = threadIdx.x >> 6;
@@ -56,42 +99,20 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     if (q_gamma != nullptr) q_inv = 1.0f / sqrtf(q_sum / (float)q_cols + eps);
     if (k_gamma != nullptr) k_inv = 1.0f / sqrtf(k_sum / (float)k_cols + eps);
   }
-  const int logical = pos / page_size;
-  int page = -1;
-  if (logical < table_width) page = tables[(int64_t)tok_item[t] * table_width + logical];
-  const bool stored = page >= 0 && page < num_pages;
-  const int offset = pos - logical * page_size;
-  const int half = cache_dim / 2;   // cache_dim is even
-  // queries and keys, a pair of neighbouring dimensions per thread and turn
-  const int q_pairs = heads * half, k_pairs = kv_heads * half;
-  for (int i = threadIdx.x; i < q_pairs + k_pairs; i += blockDim.x) {
-    const bool is_q = i < q_pairs;
-    const int j = is_q ? i : i - q_pairs;
-    const int head = j / half;
-    const int d0 = (j - head * half) * 2;
-    const int src = (is_q ? q_col : k_col) + head * key_dim + d0;
-    const float* gamma = is_q ? q_gamma : k_gamma;
-    const float inv = is_q ? q_inv : k_inv;
-    float a = 0.f, b = 0.f;
-    if (d0 < key_dim) a = row[src] * inv * (gamma ? gamma[head * key_dim + d0] : 1.f);
-    if (d0 + 1 < key_dim) b = row[src + 1] * inv * (gamma ? gamma[head * key_dim + d0 + 1] : 1.f);
-    if (d0 + 1 < rot_dims) {
-      const float angle = (float)pos * freqs[d0 >> 1];
-      float sn, cs;
-      sincosf(angle, &sn, &cs);
-      const float ra = a * cs - b * sn;
-      const float rb = b * cs + a * sn;
-      a = ra;
-      b = rb;
-    }
-    if (is_q) {
-      T* dst = q_out + (int64_t)t * q_stride + (int64_t)head * cache_dim + d0;
-      dst[0] = from_float<T>(a);
-      dst[1] = from_float<T>(b);
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const Pair p = i == (int)threadIdx.x ? first : load_pair(i);
+    const float inv = p.is_q ? q_inv : k_inv;
+    const float a = p.a * inv * p.wa, b = p.b * inv * p.wb;
+    const float ra = a * p.cs - b * p.sn;
+    const float rb = b * p.cs + a * p.sn;
+    if (p.is_q) {
+      T* dst = q_out + (int64_t)t * q_stride + (int64_t)p.head * cache_dim + p.d0;
+      dst[0] = from_float<T>(ra);
+      dst[1] = from_float<T>(rb);
     } else if (stored) {
-      T* dst = k_pool + (((int64_t)page * kv_heads + head) * page_size + offset) * cache_dim + d0;
-      dst[0] = from_float<T>(a);
-      dst[1] = from_float<T>(b);
+      T* dst = k_pool + (((int64_t)page * kv_heads + p.head) * page_size + offset) * cache_dim + p.d0;
+      dst[0] = from_float<T>(ra);
+      dst[1] = from_float<T>(rb);
     }
   }
   const float lambda = v_mode == 2 ? v_lambda[0] : 0.f;

@@ -42,7 +42,8 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
   }
   float sumsq = 0.f;
   float* row = X + (int64_t)t * STREAMS * width;
-  for (int col = threadIdx.x; col < width; col += blockDim.x) {
+  // what one column needs; returns its u
+  auto column = [&](const int col) -> float {
     float x[STREAMS];
 #pragma unroll
     for (int s = 0; s < STREAMS; ++s) x[s] = row[(int64_t)s * width + col];
@@ -60,14 +61,31 @@ __global__ __launch_bounds__(HS_THREADS) void hyper_step_kernel(
 #pragma unroll
       for (int s = 0; s < STREAMS; ++s) x[s] = nx[s];
     }
-    if (reads) {
-      float uu = 0.f;
+    float uu = 0.f;
 #pragma unroll
-      for (int s = 0; s < STREAMS; ++s) uu = fmaf(w_in[s], x[s], uu);
+    for (int s = 0; s < STREAMS; ++s) uu = fmaf(w_in[s], x[s], uu);
+    if (zero != nullptr) zero[(int64_t)t * width + col] = 0.f;
+    return uu;
+  };
+  if (width <= (int)blockDim.x) {
+    // a thread per column: u and the norm's scale stay in registers, and the scale's load
+    // leaves with the others instead of behind the sum of squares
+    const int col = threadIdx.x;
+    const bool active = col < width;
+    const float g = (reads && active) ? gamma[col] : 0.f;
+    const float uu = active ? column(col) : 0.f;
+    if (!reads) return;
+    const float total = block_sum(uu * uu, red);
+    const float inv = 1.0f / sqrtf(total / (float)width + eps);
+    if (active) normed[(int64_t)t * width + col] = from_float<TOut>(uu * inv * g);
+    return;
+  }
+  for (int col = threadIdx.x; col < width; col += blockDim.x) {
+    const float uu = column(col);
+    if (reads) {
       s_u[col] = uu;
       sumsq = fmaf(uu, uu, sumsq);
     }
-    if (zero != nullptr) zero[(int64_t)t * width + col] = 0.f;
   }
   if (!reads) return;
   const float total = block_sum(sumsq, red);
