@@ -29,7 +29,7 @@
 template <typename T>
 __global__ __launch_bounds__(64) void attention_reduce_kernel(
     const float* __restrict__ partial, T* __restrict__ out, int64_t out_stride,
-    const int* __restrict__ tok_list, int heads, int head_dim, int splits) {
+    const int* __restrict__ tok_list, int heads, int head_dim, int splits, const AttnExtras extra) {
   const int n = blockIdx.x;
   const int head = blockIdx.y;
   const int lane = threadIdx.x;
@@ -41,6 +41,7 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(
   const float total_m = wave_max(m_s);
   const float weight = (m_s == -INFINITY) ? 0.f : exp2_fast<T>(m_s - total_m);
   const float total_l = wave_sum(l_s * weight);
+  const float gate = gate_factor(extra, t, head);
   // Every lane takes part in every round, also where head_dim leaves it no dimension: the
   // weights travel by shuffles, and a shuffle only reads lanes that execute it.
   for (int d0 = 0; d0 < head_dim; d0 += 64) {
@@ -51,7 +52,7 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(
     for (int s = 0; s < splits; ++s)
       value = fmaf(src[s * stride + safe_d], __shfl(weight, s, 64), value);
     if (mine)
-      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / total_l);
+      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / total_l * gate);
   }
 }
 
@@ -61,7 +62,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
                          const int* tok_item, const int* tok_pos, const int* tables,
                          int table_width, int count, int heads, int kv_heads, int head_dim,
                          int page_size, int num_pages, float scale, int window, int splits,
-                         int waves, const float* sink, hipStream_t s) {
+                         int waves, const AttnExtras extra, hipStream_t s) {
   int page_shift = -1;
   if ((page_size & (page_size - 1)) == 0) {
     page_shift = 0;
@@ -74,7 +75,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
                      (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,         \
                      out_stride, partial, tok_list, tok_item, tok_pos, tables, table_width,      \
                      heads, kv_heads, head_dim, page_size, page_shift, num_pages,                \
-                     scale * 1.4426950408889634f, window, splits, sink)
+                     scale * 1.4426950408889634f, window, splits, extra)
   // more blocks than compute units: the step is bound by memory bandwidth, not by one round trip
   const bool streaming = sizeof(T) == 2 && (int64_t)count * heads * splits > ps_compute_units();
 #define PS_LAUNCH_ADW(LPK, WAVES)          \
@@ -105,7 +106,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
   PS_CHECK_LAUNCH("ps_attention_decode");
   if (splits > 1 && out != nullptr) {
     hipLaunchKernelGGL(attention_reduce_kernel<T>, dim3(count, heads), dim3(64), 0, s, partial,
-                       (T*)out, out_stride, tok_list, heads, head_dim, splits);
+                       (T*)out, out_stride, tok_list, heads, head_dim, splits, extra);
     PS_CHECK_LAUNCH("ps_attention_decode(reduce)");
   }
   return 0;
@@ -196,10 +197,10 @@ extern "C" int ps_attention_decode_static(const void* q, int64_t q_stride, const
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, nullptr, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{nullptr, nullptr, 0}, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, nullptr, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{nullptr, nullptr, 0}, s);
 }
 
 // The partial records only (see pagedserve_hip.h).
@@ -222,10 +223,10 @@ extern "C" int ps_attention_decode_partial(const void* q, int64_t q_stride, cons
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, nullptr, 0}, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, nullptr, 0}, s);
 }
 
 extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool,
@@ -234,8 +235,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
                                    const int* tok_item, const int* tok_pos, const int* tables,
                                    int table_width, int count, int heads, int kv_heads,
                                    int head_dim, int page_size, int num_pages, float scale,
-                                   int window, int splits, int waves, const float* sink, int dtype,
-                                   void* stream) {
+                                   int window, int splits, int waves, const float* sink,
+                                   const float* gate, int64_t gate_ld, int dtype, void* stream) {
   if (check_decode_sizes("ps_attention_decode", count, heads, kv_heads, head_dim, page_size,
                          num_pages, table_width, window, splits, waves, dtype))
     return 1;
@@ -251,8 +252,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, gate, gate_ld}, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, waves, sink, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, AttnExtras{sink, gate, gate_ld}, s);
 }

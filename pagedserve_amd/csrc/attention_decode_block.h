@@ -102,7 +102,7 @@ __device__ __forceinline__ void attention_decode_block(
     const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
     int page_size, int page_shift, int num_pages, float scale_log2, int window, int splits,
-    const float* __restrict__ sink) {
+    const AttnExtras extra) {
   constexpr int GROUPS = 64 / LPK;               // keys per wave load
   constexpr int KEYS_PER_WAVE = GROUPS * AD_UNROLL;
   float (&s_acc)[AD_WAVES][256] = lds.acc;
@@ -144,9 +144,9 @@ __device__ __forceinline__ void attention_decode_block(
                      : 0.f;
 
   float m = -INFINITY, l = 0.f;
-  if (sink != nullptr && split == 0 && wave == 0 && group == 0) {
+  if (extra.sink != nullptr && split == 0 && wave == 0 && group == 0) {
     // a score without key or value (not scaled): it starts the denominator of one lane group
-    m = sink[head] * 1.4426950408889634f;
+    m = extra.sink[head] * 1.4426950408889634f;
     l = 1.f;
   }
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -264,7 +264,8 @@ __device__ __forceinline__ void attention_decode_block(
   }
   if (splits == 1 && out != nullptr) {
     if (d < head_dim)
-      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / block_l);
+      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] =
+          from_float<T>(value / block_l * gate_factor(extra, t, head));
   } else {
     float* dst = partial + (((int64_t)n * heads + head) * splits + split) * (head_dim + 2);
     if (d < head_dim) dst[d] = value;
@@ -283,11 +284,11 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
     int page_size, int page_shift, int num_pages, float scale_log2, int window, int splits,
-    const float* __restrict__ sink) {
+    const AttnExtras extra) {
   __shared__ DecodeLds<AD_WAVES> lds;
   attention_decode_block<T, LPK, AD_WAVES, AD_UNROLL, NT>(
       lds, blockIdx.x, blockIdx.y, blockIdx.z, q, q_stride, k_pool, v_pool, out, out_stride, partial,
       tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads, head_dim, page_size,
-      page_shift, num_pages, scale_log2, window, splits, sink);
+      page_shift, num_pages, scale_log2, window, splits, extra);
 }
 

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(64 * AM_WAVES) void attention_mixed_kernel(
     const int* __restrict__ cu_tokens, const int* __restrict__ kv_lens,
     // both
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int page_size,
-    int page_shift, int num_pages, float scale, int window, const float* __restrict__ sink) {
+    int page_shift, int num_pages, float scale, int window, const AttnExtras extra) {
   typedef PrefillLds<NDB, 2, 2, 1> TileLds;
   union Lds {
     TileLds tiles;
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(64 * AM_WAVES) void attention_mixed_kernel(
     attention_decode_block<bf16_t, LPK, AM_WAVES, AM_UNROLL, NT>(
         lds.decode, n, head, 0, q, q_stride, k_pool, v_pool, out, out_stride, nullptr, tok_list,
         tok_item, tok_pos, tables, table_width, heads, kv_heads, NDB * 16, page_size, page_shift,
-        num_pages, scale * 1.4426950408889634f, window, 1, sink);
+        num_pages, scale * 1.4426950408889634f, window, 1, extra);
   } else {
     // heads fastest, as in the tiled kernel's own grid: the tiles that see the most keys first
     const int rest = block - decode_blocks;
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(64 * AM_WAVES) void attention_mixed_kernel(
     attention_prefill_block<NDB, 2, 2, 1>(lds.tiles, head, tile_index, q, q_stride, k_pool, v_pool, out,
                                           out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,
                                           table_width, heads, kv_heads, page_size, page_shift,
-                                          num_pages, scale, window, sink);
+                                          num_pages, scale, window, extra);
   }
 }
 
@@ -75,7 +75,8 @@ extern "C" int ps_attention_mixed(const void* q, int64_t q_stride, const void* k
                                   int tiles, const int* cu_tokens, const int* kv_lens,
                                   const int* tables, int table_width, int heads, int kv_heads,
                                   int head_dim, int page_size, int num_pages, float scale,
-                                  int window, const float* sink, int dtype, void* stream) {
+                                  int window, const float* sink, const float* gate, int64_t gate_ld,
+                                  int dtype, void* stream) {
   PS_REQUIRE(singles >= 0 && tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 &&
                  num_pages > 0 && table_width > 0,
              "ps_attention_mixed: bad sizes");
@@ -103,6 +104,7 @@ extern "C" int ps_attention_mixed(const void* q, int64_t q_stride, const void* k
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   hipStream_t s = (hipStream_t)stream;
+  const AttnExtras extra = {sink, gate, gate_ld};
   const int decode_blocks = singles * heads;
   // as the decode kernel chooses: more blocks of its kind than compute units read their keys
   // without leaving lines in the caches
@@ -113,7 +115,7 @@ extern "C" int ps_attention_mixed(const void* q, int64_t q_stride, const void* k
                      (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out, out_stride,    \
                      decode_blocks, tok_list, tok_item, tok_pos, tile_item, tile_q0, cu_tokens, \
                      kv_lens, tables, table_width, heads, kv_heads, page_size, page_shift,      \
-                     num_pages, scale, window, sink)
+                     num_pages, scale, window, extra)
 #define PS_LAUNCH_AM_NT(NDB, LPK)     \
   do {                                \
     if (streaming) {                  \

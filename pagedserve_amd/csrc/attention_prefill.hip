@@ -54,8 +54,8 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
                                     const int* cu_tokens, const int* kv_lens, const int* tables,
                                     int table_width, int heads, int kv_heads, int head_dim,
                                     int page_size, int num_pages, float scale, int window,
-                                    int max_kv_len, int query_tile, const float* sink, int dtype,
-                                    void* stream) {
+                                    int max_kv_len, int query_tile, const float* sink,
+                                    const float* gate, int64_t gate_ld, int dtype, void* stream) {
   PS_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_prefill: bad sizes");
@@ -86,6 +86,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   hipStream_t s = (hipStream_t)stream;
+  const AttnExtras extra = {sink, gate, gate_ld};
   dim3 grid(heads, tiles);
   // With few blocks, up to two per compute unit, which hold them all at once (128 registers and
   // 72 KB of LDS each), four waves along the keys shorten the longest block (2 x 1,024 tokens of
@@ -100,7 +101,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   hipLaunchKernelGGL((attention_prefill_kernel<NDB, 4, 1>), grid, dim3(256), 0, s,              \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
                      (bf16_t*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,  \
-                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window, sink)
+                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window, extra)
   // tiles of 128 queries: four waves along the queries, each with all 64 keys of a tile: a
   // block takes in half as many keys and values per score, and a wave's work per tile that
   // does not depend on the scores (addresses, waits, checks) is spread over twice as many
@@ -108,7 +109,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   hipLaunchKernelGGL((attention_prefill_kernel<NDB, 1, 4, 2>), grid, dim3(256), 0, s,           \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
                      (bf16_t*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,  \
-                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window, sink)
+                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window, extra)
   if (query_tile == AP_QUERIES * 2) {
     static_assert(AP_LARGE_HEAD_DIM == 64, "the cases below");
     switch (head_dim / 16) {
@@ -143,13 +144,13 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
                          (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,                     \
                          (const bf16_t*)v_pool, (bf16_t*)out, out_stride, tile_item, tile_q0,   \
                          cu_tokens, kv_lens, tables, table_width, heads, kv_heads, page_size,   \
-                         page_shift, num_pages, scale, window, sink);                                 \
+                         page_shift, num_pages, scale, window, extra);                                 \
     else                                                                                        \
       hipLaunchKernelGGL((attention_prefill_kernel<NDB, 2>), grid, dim3(256), 0, s,             \
                          (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,                     \
                          (const bf16_t*)v_pool, (bf16_t*)out, out_stride, tile_item, tile_q0,   \
                          cu_tokens, kv_lens, tables, table_width, heads, kv_heads, page_size,   \
-                         page_shift, num_pages, scale, window, sink);                                 \
+                         page_shift, num_pages, scale, window, extra);                                 \
   } while (0)
   switch (head_dim / 16) {
     case 1: PS_LAUNCH_AP(1); break;
@@ -166,7 +167,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   hipLaunchKernelGGL((attention_prefill_kernel<NDB, 2>), grid, dim3(256), 0, s,                 \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
                      (bf16_t*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,  \
-                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window, sink)
+                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window, extra)
     case 9: PS_LAUNCH_AP_LARGE(9); break;
     case 10: PS_LAUNCH_AP_LARGE(10); break;
     case 11: PS_LAUNCH_AP_LARGE(11); break;

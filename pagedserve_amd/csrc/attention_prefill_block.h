@@ -49,7 +49,7 @@ __device__ __forceinline__ void attention_prefill_block(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ cu_tokens, const int* __restrict__ kv_lens,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int page_size,
-    int page_shift, int num_pages, float scale, int window, const float* __restrict__ sink) {
+    int page_shift, int num_pages, float scale, int window, const AttnExtras extra) {
   constexpr int HD = NDB * 16;
   constexpr int ROW = HD * 2;                    // bytes of one key in a tile
   constexpr int CH = HD / 8;                     // 16-byte pieces per row
@@ -195,9 +195,9 @@ __device__ __forceinline__ void attention_prefill_block(
   // every exponential is one v_exp_f32; probabilities are rounded to bfloat16 right after.
   const float scale_log2 = scale * 1.4426950408889634f;
   float m = -INFINITY, l = 0.f;
-  if (sink != nullptr && wave_k == 0) {
+  if (extra.sink != nullptr && wave_k == 0) {
     // a score without key or value: it starts the denominator of the wave with the first keys
-    m = sink[head] * 1.4426950408889634f;
+    m = extra.sink[head] * 1.4426950408889634f;
     l = 1.f;
   }
   f32x16 acc[NDB32];
@@ -465,7 +465,7 @@ __device__ __forceinline__ void attention_prefill_block(
 
   // element e of an accumulator: head dimension db*32 + (e/4)*8 + half*4 + e%4 of query `sub`
   if (q_valid && l > 0.f) {
-    const float inv = 1.0f / l;
+    const float inv = gate_factor(extra, tok0 + qi, head) / l;
     bf16_t* dst = out + (int64_t)(tok0 + qi) * out_stride + (int64_t)head * HD;
 #pragma unroll
     for (int db = 0; db < NDB32; ++db)
@@ -488,11 +488,11 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ cu_tokens, const int* __restrict__ kv_lens,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int page_size,
-    int page_shift, int num_pages, float scale, int window, const float* __restrict__ sink) {
+    int page_shift, int num_pages, float scale, int window, const AttnExtras extra) {
   __shared__ PrefillLds<NDB, KS, QW, KR> lds;
   attention_prefill_block<NDB, KS, QW, KR>(lds, blockIdx.x, blockIdx.y, q, q_stride, k_pool, v_pool, out,
                                            out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,
                                            table_width, heads, kv_heads, page_size, page_shift,
-                                           num_pages, scale, window, sink);
+                                           num_pages, scale, window, extra);
 }
 

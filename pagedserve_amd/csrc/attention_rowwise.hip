@@ -23,7 +23,7 @@ __global__ __launch_bounds__(64) void attention_rowwise_kernel(
     const int* __restrict__ tok_list, const int* __restrict__ tok_item,
     const int* __restrict__ tok_pos, const int* __restrict__ tables, int table_width, int heads,
     int kv_heads, int head_dim, int page_size, int num_pages, float scale, int window,
-    const float* __restrict__ sink) {
+    const AttnExtras extra) {
   __shared__ float q_row[256];
   __shared__ float prob[64];
   __shared__ int64_t key_base[64];
@@ -42,8 +42,8 @@ __global__ __launch_bounds__(64) void attention_rowwise_kernel(
   __syncthreads();
 
   // a sink is a score without a key or a value: it only takes part in the denominator
-  float running_max = sink ? sink[head] : -INFINITY;
-  float running_sum = sink ? 1.f : 0.f;
+  float running_max = extra.sink ? extra.sink[head] : -INFINITY;
+  float running_sum = extra.sink ? 1.f : 0.f;
   float acc[AR_MAX_DIMS] = {0.f, 0.f, 0.f, 0.f};
 
   for (int k0 = first_key; k0 < end_key; k0 += 64) {
@@ -88,12 +88,13 @@ __global__ __launch_bounds__(64) void attention_rowwise_kernel(
     }
   }
 
+  const float gate = gate_factor(extra, t, head);
 #pragma unroll
   for (int d = 0; d < AR_MAX_DIMS; ++d) {
     const int dim = lane + d * 64;
     if (dim < head_dim)
       out[(int64_t)t * out_stride + (int64_t)head * head_dim + dim] =
-          from_float<T>(acc[d] / running_sum);
+          from_float<T>(acc[d] / running_sum * gate);
   }
 }
 
@@ -103,7 +104,8 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
                                     const int* tables, int table_width, int tokens, int heads,
                                     int kv_heads,
                                     int head_dim, int page_size, int num_pages, float scale,
-                                    int window, const float* sink, int dtype, void* stream) {
+                                    int window, const float* sink, const float* gate,
+                                    int64_t gate_ld, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_rowwise: bad sizes");
@@ -116,17 +118,18 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_rowwise: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  const AttnExtras extra = {sink, gate, gate_ld};
   dim3 grid(tokens, heads);
   if (dtype == PS_F32)
     hipLaunchKernelGGL(attention_rowwise_kernel<float>, grid, dim3(64), 0, s, (const float*)q,
                        q_stride, (const float*)k_pool, (const float*)v_pool, (float*)out,
                        out_stride, tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads,
-                       head_dim, page_size, num_pages, scale, window, sink);
+                       head_dim, page_size, num_pages, scale, window, extra);
   else
     hipLaunchKernelGGL(attention_rowwise_kernel<bf16_t>, grid, dim3(64), 0, s, (const bf16_t*)q,
                        q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out,
                        out_stride, tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads,
-                       head_dim, page_size, num_pages, scale, window, sink);
+                       head_dim, page_size, num_pages, scale, window, extra);
   PS_CHECK_LAUNCH("ps_attention_rowwise");
   return 0;
 }

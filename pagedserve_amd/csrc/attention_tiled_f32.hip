@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ cu_tokens, const int* __restrict__ kv_lens,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
-    int page_size, int num_pages, float scale, int window, const float* __restrict__ sink) {
+    int page_size, int num_pages, float scale, int window, const AttnExtras extra) {
   constexpr int STRIDE = 64 * DV + 4;   // floats from row to row of q, k and v in LDS
   __shared__ __attribute__((aligned(16))) float s_q[AF_TILE * STRIDE];
   __shared__ __attribute__((aligned(16))) float s_k[AF_TILE * STRIDE];
@@ -79,8 +79,8 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     // (a sink is a score without key or value: it starts the denominator)
-    run_max[i] = sink ? sink[head] : -INFINITY;
-    run_sum[i] = sink ? 1.f : 0.f;
+    run_max[i] = extra.sink ? extra.sink[head] : -INFINITY;
+    run_sum[i] = extra.sink ? 1.f : 0.f;
 #pragma unroll
     for (int v = 0; v < DV; ++v) acc[v][i] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
@@ -209,7 +209,8 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     if (q_pos[i] < 0) continue;
-    const float inverse = run_sum[i] > 0.f ? 1.f / run_sum[i] : 0.f;
+    const float inverse = (run_sum[i] > 0.f ? 1.f / run_sum[i] : 0.f) *
+                          gate_factor(extra, tok0 + q0 + 4 * ty + i, head);
     float* row = out + (int64_t)(tok0 + q0 + 4 * ty + i) * out_stride + (int64_t)head * head_dim;
 #pragma unroll
     for (int v = 0; v < DV; ++v) {
@@ -234,7 +235,8 @@ extern "C" int ps_attention_tiled_f32(const void* q, int64_t q_stride, const voi
                                       const int* cu_tokens, const int* kv_lens, const int* tables,
                                       int table_width, int heads, int kv_heads, int head_dim,
                                       int page_size, int num_pages, float scale, int window,
-                                      const float* sink, void* stream) {
+                                      const float* sink, const float* gate, int64_t gate_ld,
+                                      void* stream) {
   PS_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_tiled_f32: bad sizes");
@@ -252,11 +254,12 @@ extern "C" int ps_attention_tiled_f32(const void* q, int64_t q_stride, const voi
   PS_REQUIRE(blocks < ((int64_t)1 << 31), "ps_attention_tiled_f32: too many blocks");
   if (blocks == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  const AttnExtras extra = {sink, gate, gate_ld};
 #define PS_LAUNCH_AF(DV)                                                                          \
   hipLaunchKernelGGL(attention_tiled_f32_kernel<DV>, dim3((unsigned)blocks), dim3(256), 0, s,     \
                      (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,       \
                      (float*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,     \
-                     table_width, heads, kv_heads, head_dim, page_size, num_pages, scale, window, sink)
+                     table_width, heads, kv_heads, head_dim, page_size, num_pages, scale, window, extra)
   if (head_dim <= 64) {
     PS_LAUNCH_AF(1);
   } else {

@@ -210,6 +210,20 @@ __device__ inline float apply_activation(float v) {
   return v;
 }
 
+// What an attention kernel may be given beside its operands: a sink (one float per head whose
+// exponential joins the softmax's denominator; null: none) and a gate (the output of token t
+// and head h is multiplied by sigmoid(gate[t * gate_ld + h]); null: none).
+struct AttnExtras {
+  const float* sink;
+  const float* gate;
+  long long gate_ld;
+};
+
+__device__ inline float gate_factor(const AttnExtras& extra, long long token, int head) {
+  if (extra.gate == nullptr) return 1.f;
+  return 1.0f / (1.0f + expf(-extra.gate[token * extra.gate_ld + head]));
+}
+
 // ---- error channel -------------------------------------------------------
 void ps_set_error(const char* fmt, ...);
 

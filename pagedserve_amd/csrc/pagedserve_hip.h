@@ -115,12 +115,16 @@ int ps_kv_write(const void* k, const void* v, int64_t stride, void* k_pool, void
 // null) over their requests' cached keys 0..position (or the last `window` of them), one
 // wave per (token, head).  Any head_dim from 1 to 256; heads must be a multiple of kv_heads.
 // sink: null, or one float per head that enters the softmax's denominator as exp(sink[head])
-// (a score without key or value, not scaled); the same in the attention kernels below.
+// (a score without key or value, not scaled); gate: null, or a float per token and head, rows
+// gate_ld apart: the output of token t and head h is multiplied by sigmoid(gate[t * gate_ld + h]);
+// the same in the attention kernels below (ps_attention_decode_partial leaves the gate to
+// whoever merges its records).
 int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                          void* out, int64_t out_stride, const int* tok_list, const int* tok_item,
                          const int* tok_pos, const int* tables, int table_width, int tokens,
                          int heads, int kv_heads, int head_dim, int page_size, int num_pages,
-                         float scale, int window, const float* sink, int dtype, void* stream);
+                         float scale, int window, const float* sink, const float* gate,
+                         int64_t gate_ld, int dtype, void* stream);
 
 // The same result in true 32-bit for the items of several tokens (prompt portions), a block
 // of four waves per (tile of ps_attention_tiled_f32_tile() queries, head): float pools, float
@@ -133,7 +137,8 @@ int ps_attention_tiled_f32(const void* q, int64_t q_stride, const void* k_pool, 
                            void* out, int64_t out_stride, const int* tile_item, const int* tile_q0,
                            int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                            int table_width, int heads, int kv_heads, int head_dim, int page_size,
-                           int num_pages, float scale, int window, const float* sink, void* stream);
+                           int num_pages, float scale, int window, const float* sink, const float* gate,
+                           int64_t gate_ld, void* stream);
 
 // The same result for single queries, with each token's keys cut into `splits` ranges that
 // run as separate blocks of `waves` (4 or 16) waves; `partial` is scratch of
@@ -146,7 +151,8 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
                         const int* tok_list, const int* tok_item, const int* tok_pos,
                         const int* tables, int table_width, int count, int heads, int kv_heads,
                         int head_dim, int page_size, int num_pages, float scale, int window,
-                        int splits, int waves, const float* sink, int dtype, void* stream);
+                        int splits, int waves, const float* sink, const float* gate, int64_t gate_ld,
+                        int dtype, void* stream);
 
 // Only the records of ps_attention_decode: (unnormalised sum of values [head_dim], maximum in
 // units of log 2, sum) per (token, head, range) at partial[((n * heads + head) * splits + s) *
@@ -203,7 +209,8 @@ int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, co
                          int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                          int table_width, int heads, int kv_heads, int head_dim, int page_size,
                          int num_pages, float scale, int window, int max_kv_len, int query_tile,
-                         const float* sink, int dtype, void* stream);
+                         const float* sink, const float* gate, int64_t gate_ld, int dtype,
+                         void* stream);
 
 // Both of the above in one launch, for a step that has items of one token (tok_list lists the
 // `singles` tokens; tok_item and tok_pos are indexed by token as in ps_attention_decode, which
@@ -218,7 +225,7 @@ int ps_attention_mixed(const void* q, int64_t q_stride, const void* k_pool, cons
                        const int* tile_q0, int tiles, const int* cu_tokens, const int* kv_lens,
                        const int* tables, int table_width, int heads, int kv_heads, int head_dim,
                        int page_size, int num_pages, float scale, int window, const float* sink,
-                       int dtype, void* stream);
+                       const float* gate, int64_t gate_ld, int dtype, void* stream);
 
 // The constants of that kernel that a caller builds its index arrays by: queries per tile (of
 // the two sizes), and the widest block table (entries per item) that it takes.

@@ -33,7 +33,7 @@ _SIGNATURES = {
                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_attention_rowwise": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                             c_int, c_float, c_int, c_void_p, c_int, c_void_p],
+                             c_int, c_float, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p],
     "ps_hyper_step": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
                       c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ps_streams_expand": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -52,8 +52,8 @@ _SIGNATURES = {
     "ps_softcap": [c_void_p, c_int64, c_int, c_int, c_float, c_void_p],
     "ps_attention_decode": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                            c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int,
-                            c_void_p],
+                            c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p,
+                            c_int64, c_int, c_void_p],
     "ps_attention_decode_partial": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
@@ -61,14 +61,15 @@ _SIGNATURES = {
                                   c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
     "ps_attention_tiled_f32": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                               c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
+                               c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_int64, c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
+                             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,
+                             c_int, c_void_p],
     "ps_attention_mixed": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int,
-                           c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p,
+                           c_int64, c_int, c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -659,8 +660,19 @@ def _check_sink(sink, heads):
     return sink.data_ptr()
 
 
+def _check_gate(gate, tokens, heads):
+    """(address, row stride) of the gates: a float per token and head whose sigmoid multiplies
+    the head's output (columns of a wider float tensor), or (0, 0) for None."""
+    if gate is None:
+        return 0, 0
+    _check(gate, "gate", torch.float32, 2)
+    if gate.shape[0] < tokens or gate.shape[1] != heads:
+        raise KernelError(f"attention: gates must be float [>= {tokens}, {heads}], got {tuple(gate.shape)}")
+    return gate.data_ptr(), _rows(gate, "gate")
+
+
 def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, window=0,
-                      tok_list=None, sink=None):
+                      tok_list=None, sink=None, gate=None):
     """out[t, h] = softmax(q[t, h] . K * scale) V over the cached keys of t's request, for the
     tokens in ``tok_list`` (all when it is None).  ``sink``: one float per head whose
     exponential joins the denominator (a score that has no key and no value)."""
@@ -670,7 +682,8 @@ def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 
     _call("ps_attention_rowwise", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
           out.data_ptr(), out_stride, _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(),
           tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
-          float(scale), int(window), sink, dtype_code(q.dtype), _stream())
+          float(scale), int(window), sink, *_check_gate(gate, q.shape[0], heads), dtype_code(q.dtype),
+          _stream())
     return out
 
 
@@ -682,7 +695,7 @@ def decode_keys_per_block(head_dim: int, waves: int = 4) -> int:
 
 
 def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
-                     partial=None, window=0, tok_list=None, waves=4, sink=None):
+                     partial=None, window=0, tok_list=None, waves=4, sink=None, gate=None):
     """The same result as ``attention_rowwise`` by the split-KV kernel; ``partial`` is float
     scratch of ``count * heads * splits * (head_dim + 2)`` values when ``splits > 1``.
     ``tok_item=None`` says that token t is item t (row t of ``tables``), as in a step of single
@@ -699,7 +712,8 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
           out.data_ptr(), out_stride, _ptr(partial if splits > 1 else None), floats,
           _ptr(tok_list), _ptr(tok_item), tok_pos.data_ptr(), tables.data_ptr(),
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
-          int(window), int(splits), int(waves), _check_sink(sink, heads), dtype_code(q.dtype), _stream())
+          int(window), int(splits), int(waves), _check_sink(sink, heads),
+          *_check_gate(gate, q.shape[0], heads), dtype_code(q.dtype), _stream())
     return out
 
 
@@ -848,7 +862,7 @@ def prefill_large_tile_pays(heads, head_dim, large_tiles, max_kv_len=0) -> bool:
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
                       heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE, memo=None,
-                      shared=None, sink=None):
+                      shared=None, sink=None, gate=None):
     """Attention of items with several tokens, ``query_tile`` (64, 32 or 128) queries per block,
     on the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
     the tiles that see the most keys belong first.
@@ -859,7 +873,7 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
         step_key = ("prefill", q.data_ptr(), q.shape[0], out.data_ptr(),
                     tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
                     cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale,
-                    window, max_kv_len, query_tile, _ptr(sink))
+                    window, max_kv_len, query_tile, _ptr(sink), _ptr(gate))
         key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
         kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
@@ -889,7 +903,8 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
                 out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
                 kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
-                int(query_tile), _check_sink(sink, heads), dtype_code(q.dtype)),
+                int(query_tile), _check_sink(sink, heads), *_check_gate(gate, q.shape[0], heads),
+                dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 
@@ -904,7 +919,7 @@ _TILED_F32_CHECKED = False
 
 
 def attention_tiled_f32(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
-                        scale, window=0, sink=None):
+                        scale, window=0, sink=None, gate=None):
     """Attention of items with several tokens in true 32-bit, ``PREFILL_TILE`` queries per
     block: keys and values pass through LDS once per tile of queries instead of once per query
     (``attention_rowwise``), scores and sums are plain float arithmetic.  The tile list is the
@@ -940,7 +955,7 @@ def attention_tiled_f32(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, k
           out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
           cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
           kv_heads, head_dim, page_size, pages, float(scale), int(window), _check_sink(sink, heads),
-          _stream())
+          *_check_gate(gate, q.shape[0], heads), _stream())
     return out
 
 
@@ -992,7 +1007,7 @@ def _sibling_call(memo, shared, key, step_key, k_pool, v_pool):
 
 def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_item, tile_q0,
                     cu_tokens, kv_lens, tables, heads, scale, window=0, memo=None, shared=None,
-                    sink=None):
+                    sink=None, gate=None):
     """The attention of a step that mixes decoded tokens with prompt portions, in one launch:
     the tokens listed in ``tok_list`` (the step's one-token items) as ``attention_decode`` with
     one range of keys computes them, the tiles of 64 queries listed in ``tile_item`` /
@@ -1008,7 +1023,7 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
                     tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(), positions.data_ptr(),
                     tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
                     cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale, window,
-                    _ptr(sink))
+                    _ptr(sink), _ptr(gate))
         key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
         kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
@@ -1042,7 +1057,7 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
                 positions.data_ptr(), tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
                 kv_heads, head_dim, page_size, pages, float(scale), int(window),
-                _check_sink(sink, heads), dtype_code(q.dtype)),
+                _check_sink(sink, heads), *_check_gate(gate, q.shape[0], heads), dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 

@@ -37,7 +37,8 @@ class Attention(Mixer):
       ``(1 - l) v + l v_source`` with the learned ``value_mix.weight`` ``l`` and the source's
       values of the same token.
     * ``head_gate``: each head's output is multiplied by ``sigmoid`` of a projection of the
-      layer's input (one more row per head in the packed product, ``[q | k | v | gate]``).
+      layer's input (one more row per head in the packed product, ``[q | k | v | gate]``); the
+      attention kernels do it where they store the output.
     """
 
     graph_safe = True
@@ -179,9 +180,7 @@ class Attention(Mixer):
             v_mode=self.VALUE_MIXES.index(self.value_mix))
         return q, (proj[:, gate_col:gate_col + self.heads] if self.head_gate else None)
 
-    def _project_out(self, context, gates, residual, ctx):
-        if gates is not None:
-            kernels.head_gate(context, gates, self.heads, self.head_dim)
+    def _project_out(self, context, residual, ctx):
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
                        packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace),
                        shared=ctx.shared_calls)
@@ -199,8 +198,8 @@ class Attention(Mixer):
         if sink is not None and not kernels.SINK_IN_ALL_KERNELS:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
-                                      sink=sink)
-            return self._project_out(context, gates, residual, ctx)
+                                      sink=sink, gate=gates)
+            return self._project_out(context, residual, ctx)
         return self._attend(q, context, gates, residual, ctx, cache, tables)
 
     def _project_plain(self, x, ctx, cache, tables):
@@ -259,8 +258,8 @@ class Attention(Mixer):
                                     ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
                                     ctx.kv_lens, tables, self.heads, self.scale, self.window,
                                     memo=site_memo(self._memo_attention, ctx.workspace),
-                                    shared=ctx.shared_calls, sink=sink)
-            return self._project_out(context, gates, residual, ctx)
+                                    shared=ctx.shared_calls, sink=sink, gate=gates)
+            return self._project_out(context, residual, ctx)
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
             # still fill the chip
@@ -281,7 +280,7 @@ class Attention(Mixer):
                                      ctx.positions, tables, self.heads, self.scale, splits,
                                      partial=partial, window=self.window, waves=waves,
                                      tok_list=None if singles == tokens else ctx.single_tokens,
-                                     sink=sink)
+                                     sink=sink, gate=gates)
         whole = singles == 0
         if tiled:
             size = kernels.PREFILL_TILE
@@ -299,7 +298,7 @@ class Attention(Mixer):
                                       self.heads, self.scale, self.window,
                                       max_kv_len=ctx.max_kv_len, query_tile=size,
                                       memo=site_memo(self._memo_attention, ctx.workspace),
-                                      shared=ctx.shared_calls, sink=sink)
+                                      shared=ctx.shared_calls, sink=sink, gate=gates)
         elif singles < tokens and kernels.tiled_f32_supported(self.dtype, self.head_dim):
             # 32-bit: tiles of queries too, on plain float arithmetic.  The tiles hold the items
             # of several tokens; one-token items that the split-KV kernel did not take (a head
@@ -308,17 +307,17 @@ class Attention(Mixer):
             if tile_item.numel():
                 kernels.attention_tiled_f32(q, cache.k_pool, cache.v_pool, context, tile_item, tile_q0,
                                             ctx.cu_tokens, ctx.kv_lens, tables, self.heads, self.scale,
-                                            self.window, sink=sink)
+                                            self.window, sink=sink, gate=gates)
             if not singles and ctx.single_tokens is not None and ctx.single_tokens.numel():
                 kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                           ctx.positions, tables, self.heads, self.scale, self.window,
                                           tok_list=None if ctx.single_tokens.numel() == tokens
-                                          else ctx.single_tokens, sink=sink)
+                                          else ctx.single_tokens, sink=sink, gate=gates)
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
-                                      tok_list=None if whole else ctx.portion_tokens, sink=sink)
-        self._project_out(context, gates, residual, ctx)
+                                      tok_list=None if whole else ctx.portion_tokens, sink=sink, gate=gates)
+        self._project_out(context, residual, ctx)
 
     def _one_launch(self, singles: int, ctx, tables) -> bool:
         """Whether a step's one-token items and its items of several tokens go to the kernel

@@ -135,8 +135,11 @@ def test_sink_in_every_attention_kernel(dtype, head_dim, heads, kv_heads, page_s
     q = q.to(dtype)
     tok_item = torch.arange(count, dtype=torch.int32, device="cuda")
     tok_pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device="cuda")
+    # a gate per token and head (columns of a wider tensor): the kernels multiply a head's output by its sigmoid
+    wide = torch.randn((count, heads + 3), generator=g)
+    dgate = wide.cuda()[:, 2:2 + heads]
     expected = torch.stack([_attend_plain(q[n].float(), dense[n][0], dense[n][1], scale, sink, contexts[n] - 1)
-                            for n in range(count)])
+                            for n in range(count)]) * torch.sigmoid(wide[:, 2:2 + heads].double())[:, :, None]
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     dq = q.reshape(count, -1).cuda()
     dsink = sink.cuda()
@@ -146,12 +149,13 @@ def test_sink_in_every_attention_kernel(dtype, head_dim, heads, kv_heads, page_s
         assert torch.allclose(got, expected, atol=tol, rtol=tol), (what, float((got - expected).abs().max()))
 
     out = torch.empty_like(dq)
-    kernels.attention_rowwise(dq, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, sink=dsink)
+    kernels.attention_rowwise(dq, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, sink=dsink,
+                              gate=dgate)
     check(out, "row-wise")
     # the far key's value came out where the sink is very negative, and nearly nothing where it is large
     head = 1 % heads
     if kv_heads * (head // (heads // kv_heads)) == 0:
-        got = out.double().cpu().view(count, heads, head_dim)[0, head]
+        got = out.double().cpu().view(count, heads, head_dim)[0, head] / torch.sigmoid(wide[0, 2 + head].double())
         assert torch.allclose(got, dense[0][1][targets[0], 0].double(), atol=5e-2)
     assert float(out.double().cpu().view(count, heads, head_dim)[1:, 0].abs().max()) < 0.2
     for splits in (1, 3):
@@ -159,7 +163,7 @@ def test_sink_in_every_attention_kernel(dtype, head_dim, heads, kv_heads, page_s
             partial = torch.full((count * heads * splits * (head_dim + 2),), float("nan"), device="cuda")
             out = torch.full_like(dq, float("nan"))
             kernels.attention_decode(dq, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
-                                     partial=partial, waves=waves, sink=dsink)
+                                     partial=partial, waves=waves, sink=dsink, gate=dgate)
             check(out, f"split-KV {splits} x {waves}")
     # the same queries as the last tokens of prompt portions (every request brings all its tokens)
     if head_dim % 16 == 0 or dtype == torch.float32:
@@ -172,6 +176,10 @@ def test_sink_in_every_attention_kernel(dtype, head_dim, heads, kv_heads, page_s
         for n in range(count):
             big_q[cu[n + 1] - 1] = q[n].reshape(-1)
         big_q = big_q.cuda()
+        big_gate = torch.randn((total, heads), generator=g)
+        for n in range(count):
+            big_gate[cu[n + 1] - 1] = wide[n, 2:2 + heads]
+        big_gate = big_gate.cuda()
         tile = kernels.PREFILL_TILE
         items, firsts = [], []
         for n, length in enumerate(lengths):
@@ -198,16 +206,17 @@ def test_sink_in_every_attention_kernel(dtype, head_dim, heads, kv_heads, page_s
         out = torch.full_like(big_q, float("nan"))
         if dtype == torch.float32:
             kernels.attention_tiled_f32(big_q, k_pool, v_pool, out, tile_item, tile_q0, cu_t, kv_lens, tables,
-                                        heads, scale, sink=dsink)
+                                        heads, scale, sink=dsink, gate=big_gate)
             check_rows(out, "tiled 32-bit")
         else:
             kernels.attention_prefill(big_q, k_pool, v_pool, out, tile_item, tile_q0, cu_t, kv_lens, tables,
-                                      heads, scale, sink=dsink)
+                                      heads, scale, sink=dsink, gate=big_gate)
             check_rows(out, "tiled")
             if kernels.mixed_supported(dtype, head_dim, tables.shape[1]):
                 out = torch.full_like(big_q, float("nan"))
                 kernels.attention_mixed(big_q, k_pool, v_pool, out, single_list, item_of, position_of,
-                                        tile_item, tile_q0, cu_t, kv_lens, tables, heads, scale, sink=dsink)
+                                        tile_item, tile_q0, cu_t, kv_lens, tables, heads, scale, sink=dsink,
+                                        gate=big_gate)
                 check_rows(out, "mixed")
 
 
