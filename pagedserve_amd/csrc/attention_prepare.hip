@@ -28,6 +28,7 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     const int* __restrict__ tok_pos, const int* __restrict__ tables, int table_width, int heads,
     int kv_heads, int key_dim, int value_dim, int cache_dim, int page_size, int num_pages) {
   __shared__ float red[2][16];
+  __shared__ float s_cos[128], s_sin[128];   // the token's angles, one per rotated pair of a head
   const int t = blockIdx.x;
   const float* row = proj + (int64_t)t * ld;
   const int pos = tok_pos[t];
@@ -38,13 +39,13 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
   const bool stored = page >= 0 && page < num_pages;
   const int offset = pos - logical * page_size;
   const int half = cache_dim / 2;   // cache_dim is even
-  // Queries and keys, a pair of neighbouring dimensions per thread and turn.  A pair's values,
-  // weights and rotation do not wait for the norms: a thread loads and turns its first pair
+  // Queries and keys, a pair of neighbouring dimensions per thread and turn.  A pair's values
+  // and weights do not wait for the norms: a thread loads its first pair
   // before the block meets for the sums of squares (which the same values feed), so that a
   // step of few tokens makes one trip to memory; further pairs of a thread are read again.
   const int q_pairs = heads * half, k_pairs = kv_heads * half;
   struct Pair {
-    float a, b, wa, wb, cs, sn;
+    float a, b, wa, wb;
     int head, d0;
     bool is_q;
   };
@@ -60,12 +61,11 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     p.b = p.d0 + 1 < key_dim ? row[src + 1] : 0.f;
     p.wa = (gamma && p.d0 < key_dim) ? gamma[p.head * key_dim + p.d0] : 1.f;
     p.wb = (gamma && p.d0 + 1 < key_dim) ? gamma[p.head * key_dim + p.d0 + 1] : 1.f;
-    p.cs = 1.f;
-    p.sn = 0.f;
-    if (p.d0 + 1 < rot_dims) sincosf((float)pos * freqs[p.d0 >> 1], &p.sn, &p.cs);
     return p;
   };
   const int pairs = q_pairs + k_pairs;
+  // every head turns by the same angles: they are worked out once per token, not once per head
+  for (int i = threadIdx.x; i < rot_dims / 2; i += blockDim.x) sincosf((float)pos * freqs[i], &s_sin[i], &s_cos[i]);
   const bool has_first = (int)threadIdx.x < pairs;
   Pair first = {};
   if (has_first) first = load_pair(threadIdx.x);
@@ -98,13 +98,17 @@ __global__ __launch_bounds__(1024) void attention_prepare_kernel(
     }
     if (q_gamma != nullptr) q_inv = 1.0f / sqrtf(q_sum / (float)q_cols + eps);
     if (k_gamma != nullptr) k_inv = 1.0f / sqrtf(k_sum / (float)k_cols + eps);
+  } else {
+    __syncthreads();      // the angles
   }
   for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
     const Pair p = i == (int)threadIdx.x ? first : load_pair(i);
     const float inv = p.is_q ? q_inv : k_inv;
     const float a = p.a * inv * p.wa, b = p.b * inv * p.wb;
-    const float ra = a * p.cs - b * p.sn;
-    const float rb = b * p.cs + a * p.sn;
+    const bool turned = p.d0 + 1 < rot_dims;
+    const float cs = turned ? s_cos[p.d0 >> 1] : 1.f, sn = turned ? s_sin[p.d0 >> 1] : 0.f;
+    const float ra = a * cs - b * sn;
+    const float rb = b * cs + a * sn;
     if (p.is_q) {
       T* dst = q_out + (int64_t)t * q_stride + (int64_t)p.head * cache_dim + p.d0;
       dst[0] = from_float<T>(ra);
@@ -146,6 +150,7 @@ extern "C" int ps_attention_prepare(const float* proj, int64_t ld, int q_col, in
   PS_REQUIRE(cache_dim >= key_dim && cache_dim >= value_dim && cache_dim % 2 == 0,
              "ps_attention_prepare: cached head size %d must be even and hold keys of %d and values of %d",
              cache_dim, key_dim, value_dim);
+  PS_REQUIRE(rot_dims <= 256, "ps_attention_prepare: %d rotated dimensions, the kernel keeps angles for 256", rot_dims);
   PS_REQUIRE(rot_dims >= 0 && rot_dims <= key_dim && rot_dims % 2 == 0,
              "ps_attention_prepare: %d rotated dimensions do not fit heads of %d", rot_dims, key_dim);
   PS_REQUIRE(rot_dims == 0 || freqs != nullptr, "ps_attention_prepare: rotation without frequencies");
