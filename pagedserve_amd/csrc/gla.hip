@@ -34,8 +34,8 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(
 
 // A block (one wave) owns COLS columns of one head's state for one item of the step and walks
 // the item's tokens in order: lane = row group * COLS + column.  The state's rows are dealt to
-// the 64 / COLS row groups, RPL rows per lane, in registers; o needs the sum over the row groups
-// (lane exchanges per token).  The walk is one dependent chain per token, so a launch with few
+// the 64 / COLS row groups, RPL rows per lane, in registers; o needs the sum over the row groups,
+// which is taken through LDS once per chunk.  The walk is one dependent chain per token, so a launch with few
 // blocks takes narrow ones (4 columns, 16 row groups: a quarter of the work per lane and token,
 // four times the blocks), one with many the wide ones (16 columns, 4 row groups).  The
 // tokens' q, k and decays come GLA_CHUNK at a time (32 for key heads up to 64, fewer for larger
@@ -58,6 +58,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
   __shared__ __attribute__((aligned(16))) float s_k[GLA_CHUNK][GROUPS * PAD];
   __shared__ __attribute__((aligned(16))) float s_a[GLA_CHUNK][GROUPS * PAD];
   __shared__ float s_v[GLA_CHUNK][COLS];
+  __shared__ float s_o[GLA_CHUNK][65];     // every lane's share of o_t (rows one bank apart)
   const int item = blockIdx.x, head = blockIdx.y;
   const int lane = threadIdx.x;
   const int col = blockIdx.z * COLS + (lane % COLS);
@@ -139,22 +140,24 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
       }
       return o;
     };
-    // over the lanes with the same column: rotations inside the row of 16 lanes, then the
-    // swaps of rows and halves
-    auto finish = [&](float o, const int tt) {
-      if (COLS <= 4) o += lane_exchange<0x124>(o);     // row_ror:4
-      if (COLS <= 8) o += lane_exchange<0x128>(o);     // row_ror:8
-      o = xor_sum<16>(o);
-      o = xor_sum<32>(o);
-      if (group == 0 && has_col)
-        out[(int64_t)(base + tt) * heads * value_dim + head * value_dim + col] = o;
-    };
+    // The lanes' shares wait in LDS: the state's chain then holds no exchange between lanes,
+    // and the sums over the row groups are taken for all tokens of the chunk at once.
     if (count == GLA_CHUNK) {
-      // a whole chunk: unrolled, so that the reads and sums of neighbouring tokens overlap
+      // a whole chunk: unrolled, so that the reads of the next tokens run ahead of the chain
 #pragma unroll
-      for (int tt = 0; tt < GLA_CHUNK; ++tt) finish(token(tt), tt);
+      for (int tt = 0; tt < GLA_CHUNK; ++tt) s_o[tt][lane] = token(tt);
     } else {
-      for (int tt = 0; tt < count; ++tt) finish(token(tt), tt);
+      for (int tt = 0; tt < count; ++tt) s_o[tt][lane] = token(tt);
+    }
+    __syncthreads();
+    for (int idx = lane; idx < count * COLS; idx += 64) {
+      const int tt = idx / COLS;
+      const int c = idx - tt * COLS;
+      float sum = 0.f;
+#pragma unroll
+      for (int g = 0; g < GROUPS; ++g) sum += s_o[tt][g * COLS + c];
+      const int to = blockIdx.z * COLS + c;
+      if (to < value_dim) out[(int64_t)(base + tt) * heads * value_dim + head * value_dim + to] = sum;
     }
   }
 #pragma unroll

@@ -14,8 +14,6 @@ from .library import load_library
 
 F32 = 0
 BF16 = 1
-# whether every attention kernel takes a sink (else a layer with one runs on the row-wise kernel)
-SINK_IN_ALL_KERNELS = True
 MAX_STREAMS = 8   # copies of the residual stream that ps_hyper_step takes (csrc/streams.hip)
 
 EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2, "residual": 3, "relu2": 4}

@@ -189,17 +189,11 @@ class Attention(Mixer):
         tokens = ctx.tokens
         tables = ctx.tables[cache.group]
         gates = None
-        sink = self.sink
         if self.prepared:
             q, gates = self._project_prepared(x, ctx, cache, tables)
         else:
             q = self._project_plain(x, ctx, cache, tables)
         context = ctx.workspace.first_rows("attn", self.q_cols, self.dtype, tokens)
-        if sink is not None and not kernels.SINK_IN_ALL_KERNELS:
-            kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
-                                      ctx.positions, tables, self.heads, self.scale, self.window,
-                                      sink=sink, gate=gates)
-            return self._project_out(context, residual, ctx)
         return self._attend(q, context, gates, residual, ctx, cache, tables)
 
     def _project_plain(self, x, ctx, cache, tables):
