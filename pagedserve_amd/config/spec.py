@@ -46,16 +46,18 @@ class BlockSpec:
 
     arrangement: str
     parts: Tuple[Tuple[str, PartSpec], ...]
+    # constants of the arrangement itself (a factor on what its sublayers add, for instance)
+    params: Tuple[Tuple[str, Any], ...] = ()
 
     @staticmethod
-    def make(arrangement: str, **parts: PartSpec) -> "BlockSpec":
-        return BlockSpec(arrangement, tuple(parts.items()))
+    def make(arrangement: str, params: Optional[Mapping[str, Any]] = None, **parts: PartSpec) -> "BlockSpec":
+        return BlockSpec(arrangement, tuple(parts.items()), _freeze(params or {}))
 
     def with_part(self, name: str, spec: PartSpec) -> "BlockSpec":
         """This block with the part ``name`` replaced (or added)."""
         parts = dict(self.parts)
         parts[name] = spec
-        return BlockSpec(self.arrangement, tuple(parts.items()))
+        return BlockSpec(self.arrangement, tuple(parts.items()), self.params)
 
     def part(self, name: str) -> PartSpec:
         for key, spec in self.parts:
@@ -66,7 +68,7 @@ class BlockSpec:
 
     def __getattr__(self, name):
         # block.mixer, block.norm1, ...: the named part
-        if name.startswith("__") or name in ("arrangement", "parts"):
+        if name.startswith("__") or name in ("arrangement", "parts", "params"):
             raise AttributeError(name)
         try:
             return self.part(name)
@@ -88,6 +90,9 @@ class LayerCall:
     block: int
     cache: int
     writes_cache: bool = True
+    # >= 0: row of the model's table of pass vectors (``ModelSpec.pass_rows``) that is added to the
+    # stream of every token right before this call
+    enter: int = -1
 
 
 @dataclass(frozen=True)
@@ -110,6 +115,9 @@ class ModelSpec:
     # n * width floats): all equal to the embedding at the start, summed before the final norm;
     # the blocks' arrangements say how a sublayer reads and writes them.
     streams: int = 0
+    # rows of a table ``[pass_rows, width]`` of vectors that calls of the run order may add to the
+    # stream before they run (``LayerCall.enter``); 0: the model has none
+    pass_rows: int = 0
 
     def __post_init__(self):
         if not self.blocks:
@@ -122,6 +130,10 @@ class ModelSpec:
                 raise ValueError(f"run order names block {call.block}, model has {len(self.blocks)}")
             if call.cache < 0:
                 raise ValueError("cache entries are numbered from 0")
+            if call.enter >= self.pass_rows:
+                raise ValueError(f"a call adds pass vector {call.enter}, the model has {self.pass_rows}")
+            if call.enter >= 0 and self.streams:
+                raise ValueError("pass vectors are added to a single residual stream only")
             if call.writes_cache:
                 if call.cache in writers:
                     raise ValueError(f"cache entry {call.cache} has two writers")

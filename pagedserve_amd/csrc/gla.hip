@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
     const float* __restrict__ proj, int64_t ld, int q_col, int k_col, int v_col,
     const float* __restrict__ alpha, float* __restrict__ state, float* __restrict__ out,
     const int* __restrict__ cu_tokens, const int* __restrict__ slots, int heads, int key_dim,
-    int value_dim, float q_scale) {
+    int value_dim, float q_scale, const float* __restrict__ head_decay, int silu_inputs) {
   constexpr int GROUPS = 64 / COLS;                // row groups
   constexpr int ROWS = GROUPS * RPL;               // rows with padding up to the lanes' share
   constexpr int PAD = RPL + 4;                     // row groups start in different banks
@@ -75,6 +75,8 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
   }
   const int channels = heads * key_dim;
   float rq[PER], rk[PER], ra[PER], rv[PER_V];
+  // one decay per head for all key channels and tokens (then no array of decays is read)
+  const float fixed_decay = head_decay ? head_decay[head] : 0.f;
   // every load is unconditional from a clamped address; what lies outside is masked when stored
   auto fetch = [&](const int base) {
     const int count = (t1 - base) < GLA_CHUNK ? (t1 - base) : GLA_CHUNK;
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
       const int c = head * key_dim + (r < key_dim ? r : 0);
       rq[j] = proj[t * ld + q_col + c];
       rk[j] = proj[t * ld + k_col + c];
-      ra[j] = alpha[t * channels + c];
+      ra[j] = head_decay ? fixed_decay : alpha[t * channels + c];
     }
 #pragma unroll
     for (int j = 0; j < PER_V; ++j) {
@@ -107,6 +109,10 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
       const int r = idx - tt * ROWS;
       const bool valid = tt < count && r < key_dim;
       const int at = (r / RPL) * PAD + (r % RPL);
+      if (silu_inputs) {
+        rq[j] = rq[j] / (1.0f + expf(-rq[j]));
+        rk[j] = rk[j] / (1.0f + expf(-rk[j]));
+      }
       s_q[tt][at] = valid ? rq[j] * q_scale : 0.f;
       s_k[tt][at] = valid ? rk[j] : 0.f;
       s_a[tt][at] = valid ? ra[j] : 0.f;
@@ -117,6 +123,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
       if (idx < GLA_CHUNK * COLS) {
         const int tt = idx / COLS;
         const int c = blockIdx.z * COLS + (idx - tt * COLS);
+        if (silu_inputs) rv[j] = rv[j] / (1.0f + expf(-rv[j]));
         s_v[tt][idx - tt * COLS] = (tt < count && c < value_dim) ? rv[j] : 0.f;
       }
     }
@@ -185,6 +192,42 @@ __global__ __launch_bounds__(64) void gla_output_kernel(
   }
 }
 
+// out[t, :] = o[t, :] / sqrt(mean(o[t, :]^2) + eps) * w * sigmoid(gate[t, :]): the norm over the
+// whole row (all heads together), a block per token.
+template <typename T>
+__global__ __launch_bounds__(256) void row_norm_gate_kernel(
+    const float* __restrict__ o, const float* __restrict__ w, float eps,
+    const float* __restrict__ gate, int64_t gate_ld, T* __restrict__ out, int64_t out_stride,
+    int columns) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const float* row = o + (int64_t)t * columns;
+  float sum = 0.f;
+  for (int d = threadIdx.x; d < columns; d += blockDim.x) sum = fmaf(row[d], row[d], sum);
+  const float inv = 1.0f / sqrtf(block_sum(sum, scratch) / (float)columns + eps);
+  for (int d = threadIdx.x; d < columns; d += blockDim.x) {
+    const float g = gate[(int64_t)t * gate_ld + d];
+    out[(int64_t)t * out_stride + d] = from_float<T>(row[d] * inv * w[d] / (1.0f + expf(-g)));
+  }
+}
+
+extern "C" int ps_row_norm_gate(const float* o, const float* w, float eps, const float* gate,
+                                int64_t gate_ld, void* out, int64_t out_stride, int tokens,
+                                int columns, int dtype, void* stream) {
+  PS_REQUIRE(tokens >= 0 && columns > 0 && eps > 0.f, "ps_row_norm_gate: bad sizes");
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_row_norm_gate: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    hipLaunchKernelGGL(row_norm_gate_kernel<float>, dim3(tokens), dim3(256), 0, s, o, w, eps, gate,
+                       gate_ld, (float*)out, out_stride, columns);
+  else
+    hipLaunchKernelGGL(row_norm_gate_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, o, w, eps, gate,
+                       gate_ld, (bf16_t*)out, out_stride, columns);
+  PS_CHECK_LAUNCH("ps_row_norm_gate");
+  return 0;
+}
+
 extern "C" int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank, const void* w,
                             const float* bias, float tau, float* alpha, int tokens, int channels,
                             int dtype, void* stream) {
@@ -207,7 +250,9 @@ extern "C" int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank
 extern "C" int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
                            const float* alpha, float* state, float* out, const int* cu_tokens,
                            const int* slots, int items, int max_slots, int heads, int key_dim,
-                           int value_dim, float q_scale, int longest, void* stream) {
+                           int value_dim, float q_scale, int longest, const float* head_decay,
+                           int silu_inputs, void* stream) {
+  PS_REQUIRE(alpha != nullptr || head_decay != nullptr, "ps_gla_scan: no decays given");
   PS_REQUIRE(items >= 0 && heads > 0 && key_dim > 0 && value_dim > 0 && max_slots > 0,
              "ps_gla_scan: bad sizes");
   PS_REQUIRE(key_dim <= 256, "ps_gla_scan: key head size %d above 256", key_dim);
@@ -223,7 +268,7 @@ extern "C" int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, 
   hipLaunchKernelGGL((gla_scan_kernel<RPL, COLS, CHUNK>),                                         \
                      dim3(items, heads, (value_dim + COLS - 1) / COLS),                           \
                      dim3(64), 0, s, proj, ld, q_col, k_col, v_col, alpha, state, out, cu_tokens, \
-                     slots, heads, key_dim, value_dim, q_scale)
+                     slots, heads, key_dim, value_dim, q_scale, head_decay, silu_inputs)
 #define PS_LAUNCH_GLA(RPL, COLS)                                                                  \
   do {                                                                                            \
     if (brief) {                                                                                  \

@@ -289,11 +289,16 @@ int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank, const voi
 // slots[i]) and head: S = diag(alpha_t) S + k_t v_t^T, out[t] = S^T (q_t * q_scale), token after
 // token; state: [max_slots, heads, key_dim, value_dim] float, read at the start and written
 // back at the end; out: [tokens, heads * value_dim] float.  longest: no item brings more
-// tokens than that (0: unknown); it only steers the launch shape.
+// tokens than that (0: unknown); it only steers the launch shape.  head_decay (or null): one
+// decay per head that stands for all its key channels and all tokens (alpha is then not read).
+// silu_inputs: q, k and v pass silu on their way in.
 int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
                 const float* alpha, float* state, float* out, const int* cu_tokens,
                 const int* slots, int items, int max_slots, int heads, int key_dim, int value_dim,
-                float q_scale, int longest, void* stream);
+                float q_scale, int longest, const float* head_decay, int silu_inputs, void* stream);
+// out[t, :] = rms_norm(o[t, :]) * w * sigmoid(gate[t * gate_ld ...]) over the whole row.
+int ps_row_norm_gate(const float* o, const float* w, float eps, const float* gate, int64_t gate_ld,
+                     void* out, int64_t out_stride, int tokens, int columns, int dtype, void* stream);
 // out[t, h, :] = rms_norm(o[t, h, :]) * w * silu(gate[t * gate_ld + h * value_dim ...]).
 int ps_gla_output(const float* o, const float* w, float eps, const float* gate, int64_t gate_ld,
                   void* out, int64_t out_stride, int tokens, int heads, int value_dim, int dtype,
@@ -301,6 +306,53 @@ int ps_gla_output(const float* o, const float* w, float eps, const float* gate, 
 
 // logits[r, :vocab] = cap * tanh(logits[r, :vocab] / cap), rows ld floats apart.
 int ps_softcap(float* logits, int64_t ld, int rows, int vocab, float cap, void* stream);
+
+// ---- selective state-space mixer -------------------------------------------------------------
+// state: [slots, channels, states + taps - 1] float per request: the recurrence's numbers of a
+// channel and behind them its last taps - 1 raw inputs, oldest first.
+// x[t, c] = silu(bias[c] + sum_j w[c, j] u[t - taps + 1 + j, c]) with u = proj[:, u_col + c]; inputs
+// from before the step come from the slot.
+int ps_conv_silu(const float* proj, int64_t ld, int u_col, const float* w, const float* bias,
+                 const float* state, int states, void* x, const int* tok_item,
+                 const int* cu_tokens, const int* slots, int tokens, int channels, int taps,
+                 int dtype, void* stream);
+// dt[t, c] = softplus(bias[c] + sum_r low[t * ld + r] w[c, r]) in float.
+int ps_step_size(const float* low, int64_t ld, int rank, const void* w, const float* bias, float* dt,
+                 int tokens, int channels, int dtype, void* stream);
+// Per item and channel, token after token: S[n] = exp(dt A[n]) S[n] + dt x B_t[n] with
+// A = -exp(a_log[c, n]); y = (sum_n S[n] C_t[n] + skip[c] x) * silu(z) with z = proj[:, z_col + c].
+// B and C: bc[t * bc_ld + b_col / c_col + n].  Writes the states and the last raw inputs back.
+int ps_selective_scan(const void* x, const float* dt, const float* bc, int64_t bc_ld, int b_col,
+                      int c_col, const float* proj, int64_t ld, int u_col, int z_col,
+                      const float* a_log, const float* skip, float* state, void* y,
+                      const int* cu_tokens, const int* slots, int items, int channels, int states,
+                      int taps, int dtype, void* stream);
+
+// ---- a stream whose sublayers add into a scratch row ------------------------------------------
+// h += factor * y + bias (y, bias: null for none); zero[...] = 0 (may be y); if gamma:
+// normed = h / sqrt(mean(h^2) + eps) * gamma.
+int ps_stream_step(float* h, const float* y, float factor, const float* bias, const float* gamma,
+                   float eps, void* normed, float* zero, int tokens, int width, int out_dtype,
+                   void* stream);
+// out[t, c] = silu(gu[t * ld + c]) * gu[t * ld + inner + c].
+int ps_silu_gate(const float* gu, int64_t ld, void* out, int64_t out_ld, int tokens, int inner,
+                 int dtype, void* stream);
+// y += share * (rms_norm(a) * wa + rms_norm(b) * wb) over rows of width floats; a and b are cleared.
+int ps_pair_norm_mix(float* a, float* b, const float* wa, const float* wb, float eps, float share,
+                     float* y, int tokens, int width, void* stream);
+
+// ---- mixture of experts ------------------------------------------------------------------------
+// ids / weights [tokens, top]: the experts that each row of x chooses and s * scale of each
+// (softmax over all experts of the 32-bit logits w x; only experts of the keep best of groups
+// equal groups of neighbours, a group's score being its largest s).
+int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tokens, int width, int experts,
+                 int groups, int keep, int top, float scale, int* ids, float* weights, int dtype,
+                 void* stream);
+// y[t] += sum_j weights[t, j] W2[e] (silu(W1[e][:inner] x_t) * (W1[e][inner:] x_t)), e = ids[t, j];
+// w1: [experts, 2 * inner, width], w2: [experts, width, inner]; hidden: [tokens * top, inner] scratch.
+int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2, const int* ids,
+                   const float* weights, void* hidden, float* y, int tokens, int width, int inner,
+                   int top, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

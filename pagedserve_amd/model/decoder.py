@@ -15,7 +15,8 @@ from ..config.spec import ModelSpec
 from ..ops import kernels
 from ..parts import (ARRANGEMENTS, EMBEDDINGS, HEADS, NORMS, POSITIONS, ROLES, CacheView,
                      PagedKVSpec, SlotStateSpec, build_part)
-from ..weights.loader import ParamSpec
+from ..parts.block import STREAM_BIAS
+from ..weights.loader import VECTOR, ParamSpec
 
 
 class DecoderModel:
@@ -47,7 +48,8 @@ class DecoderModel:
             if unknown:
                 raise KeyError(f"arrangement {block_spec.arrangement!r} has no part named "
                                f"{', '.join(unknown)}; it has: {', '.join(arrangement.roles)}")
-            self.blocks.append(arrangement(width=spec.width, dtype=dtype, parts=parts))
+            self.blocks.append(arrangement(width=spec.width, dtype=dtype, parts=parts,
+                                           **dict(block_spec.params)))
         self.final_norm = build_part(NORMS, "norm", spec.final_norm, **common)
         # Queries of a prompt portion are handed to the mixers in tiles; each mixer says which
         # size (or sizes) its kernel takes, and the step lists the tiles once per size that is
@@ -63,6 +65,15 @@ class DecoderModel:
         for call in spec.schedule:
             if call.writes_cache:
                 self._entry_spec[call.cache] = self.blocks[call.block].mixer.cache_spec()
+        # a mixer made of several mixers keeps one entry per child; the cache manager knows these
+        # under numbers behind the run order's own
+        self._child_entries = {}
+        following = spec.num_cache_entries
+        for entry in sorted(self._entry_spec):
+            if isinstance(self._entry_spec[entry], tuple):
+                count = len(self._entry_spec[entry])
+                self._child_entries[entry] = tuple(range(following, following + count))
+                following += count
         for call in spec.schedule:
             mine = self.blocks[call.block].mixer.cache_spec()
             if not call.writes_cache and mine != self._entry_spec[call.cache]:
@@ -75,6 +86,8 @@ class DecoderModel:
         """(prefix of the parameter paths, part) of every part that may own parameters."""
         yield "embedding.", self.embedding
         yield "position.", self.position
+        if self.spec.pass_rows:
+            yield "", self
         for index, block in enumerate(self.blocks):
             for part_name, part in block.parts().items():
                 yield f"blocks.{index}.{part_name}.", part
@@ -82,11 +95,21 @@ class DecoderModel:
         yield "head.", self.head
 
     def parameters(self) -> Dict[str, ParamSpec]:
-        return {prefix + name: spec for prefix, part in self._named_parts()
-                for name, spec in part.parameters().items()}
+        found = {}
+        for prefix, part in self._named_parts():
+            if part is self:
+                found["pass_table"] = ParamSpec((self.spec.pass_rows, self.spec.width), VECTOR)
+                continue
+            for name, spec in part.parameters().items():
+                found[prefix + name] = spec
+        return found
 
     def bind(self, tensors: Dict[str, torch.Tensor]):
         for prefix, part in self._named_parts():
+            if part is self:
+                self.pass_table = tensors["pass_table"]
+                self.pass_rows = [self.pass_table[row] for row in range(self.spec.pass_rows)]
+                continue
             mine = {name: tensors[prefix + name] for name in part.parameters()}
             if part is self.head:
                 # a tied head is the token table itself, not a copy
@@ -103,8 +126,14 @@ class DecoderModel:
         """Cache groups (entries of equal geometry share a pool) and state tensors."""
         by_geometry: Dict[tuple, List[int]] = {}
         states = []
+        flat = []
         for entry in sorted(self._entry_spec):
             spec = self._entry_spec[entry]
+            if isinstance(spec, tuple):
+                flat.extend(zip(self._child_entries[entry], spec))
+            else:
+                flat.append((entry, spec))
+        for entry, spec in flat:
             if isinstance(spec, PagedKVSpec):
                 by_geometry.setdefault((spec.kv_heads, spec.head_dim, spec.window, spec.value_dim),
                                        []).append(entry)
@@ -118,15 +147,24 @@ class DecoderModel:
 
     def cache_views(self, cache) -> List[CacheView]:
         """One view per call of the run list, in order."""
+        def view_of(entry, spec, writes):
+            view = CacheView(entry=entry, writes=writes)
+            if isinstance(spec, PagedKVSpec):
+                view.group = cache.entry_group(entry)
+                view.k_pool, view.v_pool = cache.entry_pools(entry)
+            elif isinstance(spec, SlotStateSpec):
+                view.state = cache.state(entry)
+            return view
+
         views = []
         for call in self.spec.schedule:
             spec = self._entry_spec[call.cache]
-            view = CacheView(entry=call.cache, writes=call.writes_cache)
-            if isinstance(spec, PagedKVSpec):
-                view.group = cache.entry_group(call.cache)
-                view.k_pool, view.v_pool = cache.entry_pools(call.cache)
-            elif isinstance(spec, SlotStateSpec):
-                view.state = cache.state(call.cache)
+            if isinstance(spec, tuple):
+                view = CacheView(entry=call.cache, writes=call.writes_cache)
+                view.children = [view_of(entry, child, call.writes_cache)
+                                 for entry, child in zip(self._child_entries[call.cache], spec)]
+            else:
+                view = view_of(call.cache, spec, call.writes_cache)
             views.append(view)
         return views
 
@@ -158,6 +196,15 @@ class DecoderModel:
         schedule = self.spec.schedule
         for index, (call, view) in enumerate(zip(schedule, views)):
             block = self.blocks[call.block]
+            if call.enter >= 0:
+                # the pass vector: a block that folds it into its first launch takes it, else a
+                # launch of its own adds it
+                if getattr(block, "takes_stream_bias", False):
+                    if ctx.extra is None:
+                        ctx.extra = {}
+                    ctx.extra[STREAM_BIAS] = self.pass_rows[call.enter]
+                else:
+                    kernels.stream_step(h, tokens, width, bias=self.pass_rows[call.enter])
             block.forward(h, ctx, view)
             # a block may leave its last write to the block that follows, if that one takes it
             if hasattr(block, "finish"):

@@ -44,7 +44,26 @@ _SIGNATURES = {
     "ps_gla_decay": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int,
                      c_int, c_int, c_void_p],
     "ps_gla_scan": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int,
+                    c_void_p],
+    "ps_row_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
+                         c_int, c_int, c_void_p],
+    "ps_conv_silu": [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_step_size": [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                     c_void_p],
+    "ps_selective_scan": [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+                          c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_stream_step": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                       c_int, c_int, c_int, c_void_p],
+    "ps_silu_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
+    "ps_pair_norm_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_int,
+                         c_int, c_void_p],
+    "ps_moe_route": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                     c_void_p, c_void_p, c_int, c_void_p],
+    "ps_moe_experts": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                       c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_gla_output": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
                       c_int, c_int, c_int, c_void_p],
     "ps_softcap": [c_void_p, c_int64, c_int, c_int, c_float, c_void_p],
@@ -1191,16 +1210,23 @@ def gla_decay(proj, low_col, w, bias, tau, alpha):
 
 
 def gla_scan(proj, columns, alpha, state, out, cu_tokens, slots, heads, key_dim, value_dim, q_scale,
-             longest=0):
+             longest=0, head_decay=None, silu_inputs=False):
     """The recurrence of gated linear attention over the step's items, token after token
     (``csrc/pagedserve_hip.h: ps_gla_scan``); ``state``: float ``[slots, heads, key_dim, value_dim]``.
-    ``longest``: no item brings more tokens than that (0: unknown); it steers the launch shape only."""
+    ``longest``: no item brings more tokens than that (0: unknown); it steers the launch shape only.
+    ``head_decay``: float ``[heads]``, one decay per head for all its key channels and all tokens
+    (``alpha`` is then ``None``).  ``silu_inputs``: queries, keys and values pass silu first."""
     _check(proj, "proj", torch.float32, 2)
     tokens = proj.shape[0]
     q_col, k_col, v_col = columns
     if max(q_col + heads * key_dim, k_col + heads * key_dim, v_col + heads * value_dim) > proj.shape[1]:
         raise KernelError("gla_scan: the projection's rows are too short for its columns")
-    _float_rows(alpha, "alpha", tokens, heads * key_dim)
+    if head_decay is not None:
+        _float_vector(head_decay, "head_decay", heads)
+        if alpha is not None:
+            raise KernelError("gla_scan: decays per head and per channel are both given")
+    else:
+        _float_rows(alpha, "alpha", tokens, heads * key_dim)
     _float_rows(out, "out", tokens, heads * value_dim)
     _check(state, "state", torch.float32, 4)
     if tuple(state.shape[1:]) != (heads, key_dim, value_dim) or not state.is_contiguous():
@@ -1210,9 +1236,201 @@ def gla_scan(proj, columns, alpha, state, out, cu_tokens, slots, heads, key_dim,
     items = slots.numel()
     if cu_tokens.numel() != items + 1 or not (cu_tokens.is_contiguous() and slots.is_contiguous()):
         raise KernelError("gla_scan: cu_tokens must hold one entry more than slots")
-    _call("ps_gla_scan", proj.data_ptr(), _rows(proj, "proj"), q_col, k_col, v_col, alpha.data_ptr(),
+    _call("ps_gla_scan", proj.data_ptr(), _rows(proj, "proj"), q_col, k_col, v_col, _ptr(alpha),
           state.data_ptr(), out.data_ptr(), cu_tokens.data_ptr(), slots.data_ptr(), items,
-          state.shape[0], heads, key_dim, value_dim, float(q_scale), int(longest), _stream())
+          state.shape[0], heads, key_dim, value_dim, float(q_scale), int(longest), _ptr(head_decay),
+          int(bool(silu_inputs)), _stream())
+
+
+def row_norm_gate(o, weight, eps, gate, out):
+    """``out[t] = rms_norm(o[t]) * weight * sigmoid(gate[t])``: the norm over the whole row."""
+    _check(gate, "gate", torch.float32, 2)
+    tokens, columns = gate.shape
+    _float_rows(o, "o", tokens, columns)
+    _float_vector(weight, "weight", columns)
+    _check(out, "out", ndim=2)
+    if out.shape[0] < tokens or out.shape[1] != columns:
+        raise KernelError("row_norm_gate: out must hold the gate's rows and columns")
+    _call("ps_row_norm_gate", o.data_ptr(), weight.data_ptr(), float(eps), gate.data_ptr(),
+          _rows(gate, "gate"), out.data_ptr(), _rows(out, "out"), tokens, columns,
+          dtype_code(out.dtype), _stream())
+
+
+def _step_items(cu_tokens, slots, what):
+    _check(cu_tokens, "cu_tokens", torch.int32, 1)
+    _check(slots, "slots", torch.int32, 1)
+    items = slots.numel()
+    if cu_tokens.numel() != items + 1 or not (cu_tokens.is_contiguous() and slots.is_contiguous()):
+        raise KernelError(f"{what}: cu_tokens must hold one entry more than slots")
+    return items
+
+
+def _scan_state(state, channels, states, taps, what):
+    _check(state, "state", torch.float32, 3)
+    if tuple(state.shape[1:]) != (channels, states + taps - 1) or not state.is_contiguous():
+        raise KernelError(f"{what}: state {tuple(state.shape)} must be [slots, {channels}, "
+                          f"{states + taps - 1}]")
+
+
+def conv_silu(proj, u_col, weight, bias, state, states, x, tok_item, cu_tokens, slots):
+    """``x[t, c] = silu(bias[c] + sum_j weight[c, j] u[t - taps + 1 + j, c])`` with the raw inputs
+    ``u = proj[:, u_col:u_col + channels]`` of the step and, before the step's first token of an
+    item, the inputs that the item's slot kept (``state[slot, c, states:]``, oldest first)."""
+    _check(proj, "proj", torch.float32, 2)
+    _check(weight, "weight", torch.float32, 2)
+    tokens = proj.shape[0]
+    channels, taps = weight.shape
+    if not weight.is_contiguous() or u_col + channels > proj.shape[1]:
+        raise KernelError("conv_silu: the projection's rows are too short for its channels")
+    if bias is not None:
+        _float_vector(bias, "bias", channels)
+    _scan_state(state, channels, states, taps, "conv_silu")
+    _check(x, "x", ndim=2)
+    if x.shape[0] < tokens or x.shape[1] != channels or not x.is_contiguous():
+        raise KernelError("conv_silu: x must be contiguous [>= tokens, channels]")
+    _check(tok_item, "tok_item", torch.int32, 1)
+    if tok_item.numel() < tokens:
+        raise KernelError("conv_silu: tok_item is shorter than the step")
+    _step_items(cu_tokens, slots, "conv_silu")
+    _call("ps_conv_silu", proj.data_ptr(), _rows(proj, "proj"), u_col, weight.data_ptr(), _ptr(bias),
+          state.data_ptr(), states, x.data_ptr(), tok_item.data_ptr(), cu_tokens.data_ptr(),
+          slots.data_ptr(), tokens, channels, taps, dtype_code(x.dtype), _stream())
+
+
+def step_size(low, w, bias, dt):
+    """``dt[t, c] = softplus(bias[c] + sum_r low[t, r] w[c, r])`` in float; ``low``: float columns of
+    a wider buffer."""
+    _check(low, "low", torch.float32, 2)
+    _check(w, "w", ndim=2)
+    tokens = low.shape[0]
+    channels, rank = w.shape
+    if not w.is_contiguous() or low.shape[1] != rank or low.stride(1) != 1:
+        raise KernelError("step_size: low must hold the weight's rank in columns")
+    if bias is not None:
+        _float_vector(bias, "bias", channels)
+    _float_rows(dt, "dt", tokens, channels)
+    _call("ps_step_size", low.data_ptr(), low.stride(0), rank, w.data_ptr(), _ptr(bias), dt.data_ptr(),
+          tokens, channels, dtype_code(w.dtype), _stream())
+
+
+def selective_scan(x, dt, bc, b_col, c_col, proj, u_col, z_col, a_log, skip, state, y, cu_tokens,
+                   slots, taps):
+    """The selective recurrence over the step's items (``csrc/pagedserve_hip.h: ps_selective_scan``);
+    ``state``: float ``[slots, channels, states + taps - 1]``."""
+    _check(x, "x", ndim=2)
+    tokens, channels = x.shape
+    _check(a_log, "a_log", torch.float32, 2)
+    states = a_log.shape[1]
+    if a_log.shape[0] != channels or not a_log.is_contiguous() or not x.is_contiguous():
+        raise KernelError("selective_scan: a_log must be contiguous [channels, states]")
+    _float_rows(dt, "dt", tokens, channels)
+    _float_vector(skip, "skip", channels)
+    _check(bc, "bc", torch.float32, 2)
+    _check(proj, "proj", torch.float32, 2)
+    if bc.shape[0] < tokens or max(b_col, c_col) + states > bc.shape[1] or bc.stride(1) != 1:
+        raise KernelError("selective_scan: bc is too small for the step's B and C")
+    if proj.shape[0] < tokens or max(u_col, z_col) + channels > proj.shape[1] or proj.stride(1) != 1:
+        raise KernelError("selective_scan: proj is too small for the step's inputs and gates")
+    _scan_state(state, channels, states, taps, "selective_scan")
+    _check(y, "y", x.dtype, 2)
+    if y.shape[0] < tokens or y.shape[1] != channels or not y.is_contiguous():
+        raise KernelError("selective_scan: y must be contiguous [>= tokens, channels]")
+    items = _step_items(cu_tokens, slots, "selective_scan")
+    _call("ps_selective_scan", x.data_ptr(), dt.data_ptr(), bc.data_ptr(), bc.stride(0), b_col, c_col,
+          proj.data_ptr(), proj.stride(0), u_col, z_col, a_log.data_ptr(), skip.data_ptr(),
+          state.data_ptr(), y.data_ptr(), cu_tokens.data_ptr(), slots.data_ptr(), items, channels,
+          states, taps, dtype_code(x.dtype), _stream())
+
+
+def stream_step(h, tokens, width, add=None, bias=None, norm=None, zero=None):
+    """One pass over the float stream ``h`` (``[>= tokens, width]``), every piece optional:
+    ``add = (y, factor)``: ``h += factor * y``; ``bias``: a float row added to every token;
+    ``norm = (gamma, eps, normed)``: the RMS norm of the new ``h`` times ``gamma`` goes to ``normed``
+    (engine dtype); ``zero``: a float ``[tokens, width]`` buffer that is cleared (it may be ``y``)."""
+    _float_rows(h, "h", tokens, width)
+    y, factor, gamma, eps, normed, code = None, 0.0, None, 1.0, None, F32
+    if add is not None:
+        y, factor = add
+        _float_rows(y, "y", tokens, width)
+    if bias is not None:
+        _float_vector(bias, "bias", width)
+    if norm is not None:
+        gamma, eps, normed = norm
+        _float_vector(gamma, "gamma", width)
+        _check(normed, "normed", ndim=2)
+        if normed.shape[0] < tokens or normed.shape[1] != width or not normed.is_contiguous():
+            raise KernelError("stream_step: normed must be contiguous [>= tokens, width]")
+        code = dtype_code(normed.dtype)
+    if zero is not None:
+        _float_rows(zero, "zero", tokens, width)
+    _call("ps_stream_step", h.data_ptr(), _ptr(y), float(factor), _ptr(bias), _ptr(gamma), float(eps),
+          _ptr(normed), _ptr(zero), tokens, width, code, _stream())
+
+
+def silu_gate(gu, out):
+    """``out[t, c] = silu(gu[t, c]) * gu[t, inner + c]`` for float ``gu`` of ``2 * inner`` columns."""
+    _check(gu, "gu", torch.float32, 2)
+    _check(out, "out", ndim=2)
+    tokens, inner = gu.shape[0], gu.shape[1] // 2
+    if gu.shape[1] != 2 * inner or out.shape[0] < tokens or out.shape[1] != inner:
+        raise KernelError("silu_gate: gu must hold twice out's columns")
+    _call("ps_silu_gate", gu.data_ptr(), _rows(gu, "gu"), out.data_ptr(), _rows(out, "out"), tokens,
+          inner, dtype_code(out.dtype), _stream())
+
+
+def pair_norm_mix(a, b, weight_a, weight_b, eps, share, y, tokens, width):
+    """``y += share * (rms_norm(a) * weight_a + rms_norm(b) * weight_b)``; ``a`` and ``b`` (float
+    ``[tokens, width]``) are cleared."""
+    _float_rows(a, "a", tokens, width)
+    _float_rows(b, "b", tokens, width)
+    _float_rows(y, "y", tokens, width)
+    _float_vector(weight_a, "weight_a", width)
+    _float_vector(weight_b, "weight_b", width)
+    _call("ps_pair_norm_mix", a.data_ptr(), b.data_ptr(), weight_a.data_ptr(), weight_b.data_ptr(),
+          float(eps), float(share), y.data_ptr(), tokens, width, _stream())
+
+
+def moe_route(x, router, groups, keep, top, scale, ids, weights):
+    """The experts that every row of ``x`` chooses (``ids``, int32 ``[tokens, top]``) and their
+    weights (float): softmax over all experts of the 32-bit logits, group-limited choice, the
+    scores times ``scale`` (``csrc/moe.hip``)."""
+    _check(x, "x", ndim=2)
+    _check(router, "router", torch.float32, 2)
+    tokens, width = x.shape
+    experts = router.shape[0]
+    if router.shape[1] != width or not router.is_contiguous() or x.stride(1) != 1:
+        raise KernelError("moe_route: router must be contiguous [experts, width]")
+    _check(ids, "ids", torch.int32, 2)
+    _check(weights, "weights", torch.float32, 2)
+    for tensor in (ids, weights):
+        if tensor.shape[0] < tokens or tensor.shape[1] != top or not tensor.is_contiguous():
+            raise KernelError("moe_route: ids and weights must be contiguous [>= tokens, top]")
+    _call("ps_moe_route", x.data_ptr(), x.stride(0), router.data_ptr(), tokens, width, experts,
+          int(groups), int(keep), int(top), float(scale), ids.data_ptr(), weights.data_ptr(),
+          dtype_code(x.dtype), _stream())
+
+
+def moe_experts(x, w1, w2, ids, weights, hidden, y):
+    """``y[t] += sum_j weights[t, j] W2[e] (silu(W1[e][:inner] x_t) * (W1[e][inner:] x_t))`` with
+    ``e = ids[t, j]``; ``w1``: ``[experts, 2 * inner, width]``, ``w2``: ``[experts, width, inner]``."""
+    _check(x, "x", ndim=2)
+    tokens, width = x.shape
+    _check(w1, "w1", x.dtype, 3)
+    _check(w2, "w2", x.dtype, 3)
+    experts, inner = w2.shape[0], w2.shape[2]
+    if (tuple(w1.shape) != (experts, 2 * inner, width) or tuple(w2.shape) != (experts, width, inner)
+            or not (w1.is_contiguous() and w2.is_contiguous()) or x.stride(1) != 1):
+        raise KernelError("moe_experts: w1 [experts, 2 * inner, width] and w2 [experts, width, inner] needed")
+    top = ids.shape[1]
+    _check(ids, "ids", torch.int32, 2)
+    _check(weights, "weights", torch.float32, 2)
+    _check(hidden, "hidden", x.dtype, 2)
+    if hidden.shape[0] < tokens * top or hidden.shape[1] != inner or not hidden.is_contiguous():
+        raise KernelError("moe_experts: hidden must be contiguous [>= tokens * top, inner]")
+    _float_rows(y, "y", tokens, width)
+    _call("ps_moe_experts", x.data_ptr(), x.stride(0), w1.data_ptr(), w2.data_ptr(), ids.data_ptr(),
+          weights.data_ptr(), hidden.data_ptr(), y.data_ptr(), tokens, width, inner, top,
+          dtype_code(x.dtype), _stream())
 
 
 def gla_output(o, weight, eps, gate, out, heads, value_dim):

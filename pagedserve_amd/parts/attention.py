@@ -39,6 +39,8 @@ class Attention(Mixer):
     * ``head_gate``: each head's output is multiplied by ``sigmoid`` of a projection of the
       layer's input (one more row per head in the packed product, ``[q | k | v | gate]``); the
       attention kernels do it where they store the output.
+    * ``out_bias``: whether the output projection has a bias, where that differs from ``bias``
+      (which then speaks for the packed projection alone).
     """
 
     graph_safe = True
@@ -58,7 +60,8 @@ class Attention(Mixer):
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
                  window: int = 0, bias: bool = True, value_dim: int = 0, qk_norm: bool = False,
                  norm_eps: float = 1e-6, rotary_dims: int = 0, rotary_base: float = 10000.0,
-                 sink: bool = False, value_mix: str = "none", head_gate: bool = False):
+                 sink: bool = False, value_mix: str = "none", head_gate: bool = False,
+                 out_bias=None):
         if heads % kv_heads != 0:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
         if not 0 < head_dim <= 256:
@@ -78,6 +81,8 @@ class Attention(Mixer):
         self.scale = float(scale)
         self.window = int(window)
         self.bias = bias
+        # (the output projection's bias goes with the packed projection's unless named apart)
+        self.out_has_bias = bool(bias) if out_bias is None else bool(out_bias)
         self.qk_norm = bool(qk_norm)
         self.norm_eps = float(norm_eps)
         self.rotary_dims = int(rotary_dims)
@@ -116,6 +121,7 @@ class Attention(Mixer):
         }
         if self.bias:
             params["qkv.bias"] = ParamSpec((total,), VECTOR)
+        if self.out_has_bias:
             params["out.bias"] = ParamSpec((self.width,), VECTOR)
         if self.qk_norm:
             params["q_norm.gamma"] = ParamSpec((self.heads * self.key_dim,), VECTOR)

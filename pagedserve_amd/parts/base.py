@@ -62,6 +62,8 @@ class CacheView:
     k_pool: Optional[torch.Tensor] = None      # [pages, kv_heads, page, head_dim]
     v_pool: Optional[torch.Tensor] = None      # [pages, kv_heads, page, value head size]
     state: Optional[torch.Tensor] = None       # [max_slots, ...]
+    # a mixer made of several mixers (its ``cache_spec`` is a tuple): one view per child
+    children: Optional[List["CacheView"]] = None
 
 
 class Part:
@@ -131,7 +133,8 @@ class Mixer(Part):
     accepts_pending_norm = False
 
     def cache_spec(self):
-        """``PagedKVSpec``, ``SlotStateSpec`` or ``None``."""
+        """``PagedKVSpec``, ``SlotStateSpec`` or ``None``; a mixer made of several mixers returns
+        the tuple of theirs, and each gets a cache entry of its own."""
         return None
 
     def set_position(self, position: PositionEncoding):
@@ -182,11 +185,15 @@ class Workspace:
         self.serial = next(_WORKSPACE_SERIALS)
         self._views: Dict[tuple, torch.Tensor] = {}
 
-    def rows(self, name: str, columns: int, dtype: torch.dtype, max_rows: Optional[int] = None):
+    def rows(self, name: str, columns: int, dtype: torch.dtype, max_rows: Optional[int] = None,
+             cleared: bool = False):
+        """``cleared``: the buffer holds zeros when it is made (for sums that every user leaves
+        cleared behind it)."""
         key = (name, columns, dtype, max_rows or self.max_rows)
         buffer = self._buffers.get(key)
         if buffer is None:
-            buffer = torch.empty((max_rows or self.max_rows, columns), dtype=dtype, device=self.device)
+            make = torch.zeros if cleared else torch.empty
+            buffer = make((max_rows or self.max_rows, columns), dtype=dtype, device=self.device)
             self._buffers[key] = buffer
         return buffer
 

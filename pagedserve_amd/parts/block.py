@@ -132,3 +132,69 @@ class HyperConnectedMixerBlock(HyperConnectedBlock):
     """The same with a mixer only."""
 
     roles = {"connect1": "connection", "norm1": "norm", "mixer": "mixer"}
+
+
+_SCALED_ADD = "scaled_add"    # key of ``ctx.extra``: (y, factor) of a block that is not added to the stream yet
+STREAM_BIAS = "stream_bias"   # key of ``ctx.extra``: a float row that the next block adds to every token
+
+
+@register_arrangement("parallel_scaled")
+class ParallelScaledBlock:
+    """``h += factor * (mixer(u) + feed_forward(u))`` with ``u = norm1(h)``: one norm, both
+    sublayers read its output.  The sublayers add into a float row ``y`` per token, which one
+    launch folds into the stream; that launch is the next block's first, which also adds the row
+    that the model puts before a pass (``ctx.extra[STREAM_BIAS]``), norms for the next block and
+    clears ``y`` (``kernels.stream_step``).  ``finish`` writes back where no such block follows."""
+
+    roles = {"norm1": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+    takes_stream_write = True
+    takes_stream_bias = True
+
+    def __init__(self, width, dtype, parts, factor: float = 1.0):
+        self.width = width
+        self.dtype = dtype
+        self.factor = float(factor)
+        self._parts = dict(parts)
+        self.norm1 = parts["norm1"]
+        self.mixer = parts["mixer"]
+        self.feed_forward = parts.get("feed_forward")
+        if not hasattr(self.norm1, "gamma_eps"):
+            raise ValueError("a parallel block needs an RMS norm without a shift")
+
+    @property
+    def graph_safe(self):
+        return all(getattr(part, "graph_safe", False) for part in self._parts.values())
+
+    def parts(self):
+        return dict(self._parts)
+
+    def forward(self, h, ctx, cache):
+        tokens = ctx.tokens
+        normed = ctx.workspace.first_rows("normed", self.width, self.dtype, tokens)
+        # (made cleared; every launch that folds it into the stream clears it again)
+        ctx.workspace.rows("sublayer_sum", self.width, torch.float32, cleared=True)
+        y = ctx.workspace.first_rows("sublayer_sum", self.width, torch.float32, tokens)
+        if ctx.extra is None:
+            ctx.extra = {}
+        gamma, eps = self.norm1.gamma_eps()
+        add = ctx.extra.pop(_SCALED_ADD, None)
+        kernels.stream_step(h, tokens, self.width, add=add, bias=ctx.extra.pop(STREAM_BIAS, None),
+                            norm=(gamma, eps, normed), zero=None if add is None else add[0])
+        self.mixer.forward(normed, y, ctx, cache)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(normed, y, ctx)
+        ctx.extra[_SCALED_ADD] = (y, self.factor)
+        return h
+
+    def finish(self, h, ctx):
+        """Fold in what the block left (no block follows that would)."""
+        add = ctx.extra.pop(_SCALED_ADD, None) if ctx.extra else None
+        if add is not None:
+            kernels.stream_step(h, ctx.tokens, self.width, add=add, zero=add[0])
+
+
+@register_arrangement("parallel_scaled_mixer")
+class ParallelScaledMixerBlock(ParallelScaledBlock):
+    """The same with a mixer only."""
+
+    roles = {"norm1": "norm", "mixer": "mixer"}

@@ -1,5 +1,7 @@
 """Feed-forward parts."""
 
+import torch
+
 from ..ops import kernels
 from ..weights.loader import MATRIX, VECTOR, ParamSpec
 from .base import FeedForward, site_memo
@@ -59,3 +61,102 @@ class DenseFeedForward(FeedForward):
         kernels.linear(hidden, self.down_weight, self.down_bias, residual, epilogue="residual",
                        packed=self.down_packed, a_packed=hidden_packed, memo=site_memo(self._memo_down, ctx.workspace),
                        shared=ctx.shared_calls)
+
+
+@register_feed_forward("gated")
+class GatedFeedForward(FeedForward):
+    """``residual += W_down (silu(W_gate x) * (W_up x))``, no biases.  One packed product gives
+    ``[gate | up]`` in float; the activation and the product of the halves are 32-bit."""
+
+    graph_safe = True
+
+    accepts_pending_norm = True
+
+    def __init__(self, width: int, dtype, inner: int):
+        self.width = width
+        self.dtype = dtype
+        self.inner = inner
+        self._memo_up, self._memo_down = {}, {}
+
+    def parameters(self):
+        return {
+            "gate_up.weight": ParamSpec((2 * self.inner, self.width), MATRIX),
+            "down.weight": ParamSpec((self.width, self.inner), MATRIX),
+        }
+
+    def bind(self, tensors):
+        self.gate_up_weight = tensors["gate_up.weight"]
+        self.down_weight = tensors["down.weight"]
+        self.gate_up_packed = kernels.pack_decode_weight(self.gate_up_weight)
+        self.down_packed = kernels.pack_decode_weight(self.down_weight)
+        self._memo_up.clear()
+        self._memo_down.clear()
+
+    def forward(self, x, residual, ctx):
+        tokens = ctx.tokens
+        both = ctx.workspace.first_rows("ffn_gate_up", 2 * self.inner, torch.float32, tokens)
+        kernels.linear(x, self.gate_up_weight, None, both, packed=self.gate_up_packed,
+                       memo=site_memo(self._memo_up, ctx.workspace), shared=ctx.shared_calls)
+        hidden = ctx.workspace.first_rows("ffn", self.inner, self.dtype, tokens)
+        kernels.silu_gate(both, hidden)
+        kernels.linear(hidden, self.down_weight, None, residual, epilogue="residual",
+                       packed=self.down_packed, memo=site_memo(self._memo_down, ctx.workspace),
+                       shared=ctx.shared_calls)
+
+
+@register_feed_forward("moe")
+class MixtureOfExperts(FeedForward):
+    """``experts`` small gated feed-forwards (no biases) of which each token uses ``top``:
+
+        s = softmax(W_router x) over all experts, the logits in 32-bit
+        experts form ``groups`` equal groups of neighbours; a group's score is its largest s and
+        only experts of the ``keep`` best groups may be chosen; the ``top`` largest s among them are
+        residual += sum over the chosen e of (s_e * scale) * W_down,e (silu(W_gate,e x) * (W_up,e x))
+
+    The weights are not renormalised.  The experts' matrices are stacked, ``[experts, gate rows
+    | up rows, width]`` and ``[experts, width, inner]``; the choice stays on the device
+    (``csrc/moe.hip``)."""
+
+    graph_safe = True
+
+    accepts_pending_norm = False
+
+    def __init__(self, width: int, dtype, inner: int, experts: int, top: int, groups: int = 1,
+                 keep: int = 1, scale: float = 1.0):
+        if groups < 1 or experts % groups:
+            raise ValueError(f"{groups} groups do not divide {experts} experts")
+        if not 1 <= keep <= groups:
+            raise ValueError(f"keep ({keep}) must lie in 1..groups ({groups})")
+        if not 1 <= top <= (experts // groups) * keep:
+            raise ValueError(f"top ({top}) exceeds the experts that may be chosen")
+        self.width = width
+        self.dtype = dtype
+        self.inner = inner
+        self.experts = experts
+        self.top = top
+        self.groups = groups
+        self.keep = keep
+        self.scale = float(scale)
+
+    def parameters(self):
+        return {
+            "router.weight": ParamSpec((self.experts, self.width), VECTOR),
+            "gate_up.weight": ParamSpec((self.experts * 2 * self.inner, self.width), MATRIX),
+            "down.weight": ParamSpec((self.experts * self.width, self.inner), MATRIX),
+        }
+
+    def bind(self, tensors):
+        self.router_weight = tensors["router.weight"]
+        self.gate_up_weight = tensors["gate_up.weight"].view(self.experts, 2 * self.inner, self.width)
+        self.down_weight = tensors["down.weight"].view(self.experts, self.width, self.inner)
+
+    def forward(self, x, residual, ctx):
+        tokens = ctx.tokens
+        workspace = ctx.workspace
+        ids = workspace.first_rows("moe_ids", self.top, torch.int32, tokens)
+        weights = workspace.first_rows("moe_weights", self.top, torch.float32, tokens)
+        kernels.moe_route(x, self.router_weight, self.groups, self.keep, self.top, self.scale, ids,
+                          weights)
+        hidden = workspace.rows("moe_hidden", self.inner, self.dtype,
+                                max_rows=workspace.max_rows * self.top)
+        kernels.moe_experts(x, self.gate_up_weight, self.down_weight, ids, weights, hidden, residual)

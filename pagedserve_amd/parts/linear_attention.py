@@ -95,3 +95,79 @@ class GatedLinearAttention(Mixer):
         kernels.linear(gated, self.out_weight, None, residual, epilogue="residual",
                        packed=self.out_packed, memo=site_memo(self._memo_out, workspace),
                        shared=ctx.shared_calls)
+
+
+@register_mixer("lightning_attention")
+class LightningAttention(Mixer):
+    """Linear attention with one fixed decay per head.  With ``h`` the layer's input:
+
+        q = silu(W_q h),  k = silu(W_k h),  v = silu(W_v h)        (heads x key_dim / value_dim)
+        S_t = decay_head * S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t   (per head, no other scale)
+        out = W_o (rms_norm(o) * w_norm * sigmoid(W_g h))           (the norm over all heads at once)
+
+    The state ``S`` (float, ``[heads, key_dim, value_dim]``) lives in the request's slot, starts
+    at zero and is carried from step to step.  One packed product gives ``[q | k | v | gate]`` in
+    float; the activations, the recurrence and the norm are 32-bit (``csrc/gla.hip``, the
+    recurrence kernel of gated linear attention with a decay per head)."""
+
+    graph_safe = True
+
+    accepts_pending_norm = True
+
+    def __init__(self, width: int, dtype, heads: int, key_dim: int, value_dim: int, decays,
+                 norm_eps: float):
+        if not 0 < key_dim <= 256:
+            raise ValueError(f"key_dim {key_dim} must lie in 1..256")
+        decays = tuple(float(d) for d in decays)
+        if len(decays) != heads:
+            raise ValueError(f"{len(decays)} decays for {heads} heads")
+        self.width = width
+        self.dtype = dtype
+        self.heads = heads
+        self.key_dim = key_dim
+        self.value_dim = value_dim
+        self.decays = decays
+        self.norm_eps = float(norm_eps)
+        self.k_cols = heads * key_dim
+        self.v_cols = heads * value_dim
+        self._memo_in, self._memo_out = {}, {}
+
+    def parameters(self):
+        return {
+            "in.weight": ParamSpec((2 * self.k_cols + 2 * self.v_cols, self.width), MATRIX),
+            "norm.gamma": ParamSpec((self.v_cols,), VECTOR),
+            "out.weight": ParamSpec((self.width, self.v_cols), MATRIX),
+        }
+
+    def bind(self, tensors):
+        self.in_weight = tensors["in.weight"]
+        self.norm_gamma = tensors["norm.gamma"]
+        self.out_weight = tensors["out.weight"]
+        self.head_decay = torch.tensor(self.decays, dtype=torch.float32, device=self.out_weight.device)
+        self.in_packed = kernels.pack_decode_weight(self.in_weight)
+        self.out_packed = kernels.pack_decode_weight(self.out_weight)
+        self._memo_in.clear()
+        self._memo_out.clear()
+
+    def cache_spec(self):
+        return SlotStateSpec((self.heads, self.key_dim, self.value_dim), torch.float32)
+
+    def forward(self, x, residual, ctx, cache):
+        tokens = ctx.tokens
+        k_col, v_col = self.k_cols, 2 * self.k_cols
+        gate_col = v_col + self.v_cols
+        workspace = ctx.workspace
+        proj = workspace.first_rows("lightning_proj", gate_col + self.v_cols, torch.float32, tokens)
+        kernels.linear(x, self.in_weight, None, proj, packed=self.in_packed,
+                       memo=site_memo(self._memo_in, workspace), shared=ctx.shared_calls)
+        raw = workspace.first_rows("lightning_raw", self.v_cols, torch.float32, tokens)
+        kernels.gla_scan(proj, (0, k_col, v_col), None, cache.state, raw, ctx.cu_tokens, ctx.slots,
+                         self.heads, self.key_dim, self.value_dim, 1.0,
+                         longest=1 if ctx.decode_only else 0, head_decay=self.head_decay,
+                         silu_inputs=True)
+        gated = workspace.first_rows("lightning_out", self.v_cols, self.dtype, tokens)
+        kernels.row_norm_gate(raw, self.norm_gamma, self.norm_eps,
+                              proj[:, gate_col:gate_col + self.v_cols], gated)
+        kernels.linear(gated, self.out_weight, None, residual, epilogue="residual",
+                       packed=self.out_packed, memo=site_memo(self._memo_out, workspace),
+                       shared=ctx.shared_calls)

@@ -48,6 +48,10 @@ class RMSNorm(Norm):
     def bind(self, tensors):
         self.gamma = tensors["gamma"] + self.offset if self.offset else tensors["gamma"]
 
+    def gamma_eps(self):
+        """(scale, eps) for a launch that norms along with other work on the stream."""
+        return self.gamma, self.eps
+
     def forward(self, h, out, rows=None):
         return kernels.norm(h, self.gamma, None, self.eps, out, rows=rows, rms=True)
 
