@@ -31,6 +31,7 @@ One JSON line is printed:
     python bench.py --prefill-only --steps K [--prefill-length L]   the prefill step of 2 x L tokens alone (for profiles)
     python bench.py --kernels [--shape small|medium|xl|all] [--only name,name]
     python bench.py --design kosesun [--sizes small,small_narrow,medium]   Kosesun beside GPT-2 at equal size
+    python bench.py --design zetunex [--sizes small,medium,small_many_experts]   Zetunex beside Kosesun at equal size
 
 ``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys), of
 the prefill step (2 x 1,024 tokens) and of a mixed step (32 decoded tokens beside a portion of
@@ -521,19 +522,61 @@ DESIGN_SIZES = {
 }
 
 
+def zetunex_shape(width, layers, heads, kv_heads, dim, ff, vocab, window=512, experts=8, top=2, every=4):
+    """A Zetunex configuration of a real model's layer sizes: every ``every``-th layer is lightning
+    attention, the others windowed attention beside a selective scan twice the width; layers
+    take turns between a dense feed-forward and ``experts`` experts of which ``top`` together are as
+    wide as the dense one."""
+    listed = []
+    for index in range(layers):
+        if index % every == every - 1:
+            decay = [1.0 - 2.0 ** (-1 - 7 * h / max(heads - 1, 1)) for h in range(heads)]
+            entry = {"type": "lightning", "mixer": {"heads": heads, "dim": dim, "vdim": dim, "decay": decay}}
+        else:
+            left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                    "mask": {"size": window}}
+            right = {"inner": 2 * width, "state": 16, "dt_rank": width // 16, "conv": 4}
+            entry = {"type": "parallel", "mixer": {"left": left, "right": right}}
+        if index % 2:
+            entry["mlp"] = {"kind": "moe", "expert": {"ff": ff // top},
+                            "router": {"experts": experts, "top": top, "scale": 1.0,
+                                       "groups": {"count": 2, "keep": 1}}}
+        else:
+            entry["mlp"] = {"kind": "dense", "ff": ff}
+        listed.append(entry)
+    return {"architecture": "Zetunex", "vocab": vocab, "width": width, "layers": listed,
+            "norm": {"eps": 1e-6}, "residual_mult": 0.5}
+
+
+# name -> (Zetunex configuration, the Kosesun configuration of equal width, depth, heads and inner width)
+ZETUNEX_SIZES = {
+    "small": (zetunex_shape(768, 12, 12, 4, 64, 3072, 50257), kosesun_shape(768, 12, 12, 4, 64, 64, 3072, 50257)),
+    "medium": (zetunex_shape(1024, 24, 16, 4, 64, 4096, 50257), kosesun_shape(1024, 24, 16, 4, 64, 64, 4096, 50257)),
+    # two of sixteen experts per token
+    "small_many_experts": (zetunex_shape(768, 12, 12, 4, 64, 3072, 50257, experts=16),
+                           kosesun_shape(768, 12, 12, 4, 64, 64, 3072, 50257)),
+}
+DESIGNS = {"kosesun": (("kosesun", "gpt2"), DESIGN_SIZES), "zetunex": (("zetunex", "kosesun"), ZETUNEX_SIZES)}
+
+
 def design_comparison(args):
-    """``--design kosesun``: prefill (2 x 1,024 tokens) and decode (``--batch`` requests whose
-    contexts end at 1,024) throughput of Kosesun models beside GPT-2 models of equal width,
-    depth, head count, inner width and vocabulary, random weights, same engine and scheduler."""
+    """``--design NAME``: prefill (2 x 1,024 tokens) and decode (``--batch`` requests whose
+    contexts end at 1,024) throughput of models of the design beside models of the closest
+    other design at equal width, depth, head count, inner width and vocabulary (Kosesun beside
+    GPT-2, Zetunex beside Kosesun), random weights, same engine and scheduler."""
     import torch
 
     results = {}
     context = 1024
+    labels, sizes = DESIGNS[args.design]
+    first, second = labels
     for name in [piece for piece in args.sizes.split(",") if piece]:
-        if name not in DESIGN_SIZES:
-            raise SystemExit(f"--sizes: unknown size {name!r}; known: {', '.join(DESIGN_SIZES)}")
+        if name not in sizes:
+            if args.sizes == "small,small_narrow,medium":
+                continue      # (the default list names what the first design has)
+            raise SystemExit(f"--sizes: unknown size {name!r}; known: {', '.join(sizes)}")
         entry = {}
-        for label, raw in zip(("kosesun", "gpt2"), DESIGN_SIZES[name]):
+        for label, raw in zip(labels, sizes[name]):
             pages = 64 * (context // PAGE_SIZE) + 8
             engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
                                              shape=raw, pages=pages, max_context=context)
@@ -549,10 +592,10 @@ def design_comparison(args):
             print(f"{name} {label}: {entry[label]}", file=sys.stderr, flush=True)
             del engine, sampler
             torch.cuda.empty_cache()
-        entry["prefill_ratio"] = round(entry["kosesun"]["prefill_tokens_per_s"] / entry["gpt2"]["prefill_tokens_per_s"], 3)
-        entry["decode_ratio"] = round(entry["kosesun"]["decode_tokens_per_s"] / entry["gpt2"]["decode_tokens_per_s"], 3)
+        entry["prefill_ratio"] = round(entry[first]["prefill_tokens_per_s"] / entry[second]["prefill_tokens_per_s"], 3)
+        entry["decode_ratio"] = round(entry[first]["decode_tokens_per_s"] / entry[second]["decode_tokens_per_s"], 3)
         results[name] = entry
-    return {"metric": "prefill tok/s at 2 x 1,024 tokens and decode tok/s, Kosesun beside GPT-2 of equal size",
+    return {"metric": f"prefill tok/s at 2 x 1,024 tokens and decode tok/s, {first} beside {second} of equal size",
             "unit": "tokens/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "batch": args.batch, "steps": args.steps, "context": context,
             "data": "synthetic (random weights, uniform-random prompt ids)", "sizes": results}
@@ -620,7 +663,7 @@ def main(argv=None):
     parser.add_argument("--rows", default="1,8,64", help="decode batch sizes of --kernels")
     parser.add_argument("--only", help="--kernels: only kernels whose name holds one of these (comma-separated)")
     parser.add_argument("--no-prefill", action="store_true", help="--kernels: decode tables only")
-    parser.add_argument("--design", choices=("kosesun",), default=None,
+    parser.add_argument("--design", choices=("kosesun", "zetunex"), default=None,
                         help="prefill and decode throughput of this design beside GPT-2 at equal size")
     parser.add_argument("--sizes", default="small,small_narrow,medium", help="--design: which sizes")
     args = parser.parse_args(argv)

@@ -167,6 +167,281 @@ extern "C" int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tok
   return 0;
 }
 
+
+// ---- few rows: every (token, choice) reads its expert's rows once, 16 bytes of k per lane ------
+// Eight consecutive k of a row as floats.
+template <typename T>
+__device__ inline void load8(const T* p, float (&v)[8]);
+template <>
+__device__ inline void load8<bf16_t>(const bf16_t* p, float (&v)[8]) {
+  const uint4 raw = *reinterpret_cast<const uint4*>(p);
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(words[i] << 16);
+    v[2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
+  }
+}
+template <>
+__device__ inline void load8<float>(const float* p, float (&v)[8]) {
+  const float4 lo = *reinterpret_cast<const float4*>(p);
+  const float4 hi = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+  v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+}
+
+// As moe_hidden_kernel for a width that is a multiple of 8: a wave owns ROWS hidden columns and
+// keeps the sums of their gate and up rows apart, so that 2 * ROWS loads are in flight per lane.
+template <typename T, int ROWS>
+__global__ __launch_bounds__(256) void moe_hidden_wide_kernel(
+    const T* __restrict__ x, int64_t x_ld, const T* __restrict__ w1, const int* __restrict__ ids,
+    T* __restrict__ hidden, int width, int inner) {
+  extern __shared__ float s_x[];
+  const int64_t row_index = (int64_t)blockIdx.x * gridDim.z + blockIdx.z;
+  const int e = ids[row_index];
+  const T* x_row = x + (int64_t)blockIdx.x * x_ld;
+  for (int d = threadIdx.x; d < width; d += 256) s_x[d] = to_float<T>(x_row[d]);
+  __syncthreads();
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const T* base = w1 + (int64_t)e * 2 * inner * width;
+  const int first = (blockIdx.y * 4 + wave) * ROWS;
+  if (first >= inner) return;
+  float g[ROWS], u[ROWS];
+  const T* rows_g[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    g[r] = u[r] = 0.f;
+    const int c = first + r < inner ? first + r : inner - 1;
+    rows_g[r] = base + (int64_t)c * width;
+  }
+  const int64_t up = (int64_t)inner * width;
+  for (int d = lane * 8; d < width; d += 512) {
+    float xv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xv[i] = s_x[d + i];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      float a[8], b[8];
+      load8<T>(rows_g[r] + d, a);
+      load8<T>(rows_g[r] + up + d, b);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        g[r] = fmaf(a[i], xv[i], g[r]);
+        u[r] = fmaf(b[i], xv[i], u[r]);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const float gs = wave_sum(g[r]), us = wave_sum(u[r]);
+    if (lane == 0 && first + r < inner)
+      hidden[row_index * inner + first + r] = from_float<T>(gs / (1.0f + expf(-gs)) * us);
+  }
+}
+
+// As moe_down_kernel for an inner width that is a multiple of 8.
+template <typename T, int ROWS>
+__global__ __launch_bounds__(256) void moe_down_wide_kernel(
+    const T* __restrict__ hidden, const T* __restrict__ w2, const int* __restrict__ ids,
+    const float* __restrict__ weights, float* __restrict__ y, int width, int inner, int top) {
+  extern __shared__ float s_h[];        // [top][inner]
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < top * inner; i += 256)
+    s_h[i] = to_float<T>(hidden[t * top * inner + i]);
+  __syncthreads();
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int first = (blockIdx.y * 4 + wave) * ROWS;
+  if (first >= width) return;
+  float total[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) total[r] = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const int e = ids[t * top + j];
+    const float weight = weights[t * top + j];
+    float sum[ROWS];
+    const T* rows[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      sum[r] = 0.f;
+      const int d = first + r < width ? first + r : width - 1;
+      rows[r] = w2 + ((int64_t)e * width + d) * inner;
+    }
+    for (int c = lane * 8; c < inner; c += 512) {
+      float hv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) hv[i] = s_h[j * inner + c + i];
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        float a[8];
+        load8<T>(rows[r] + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum[r] = fmaf(a[i], hv[i], sum[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) total[r] = fmaf(weight, wave_sum(sum[r]), total[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+    if (lane == 0 && first + r < width) y[t * width + first + r] += total[r];
+}
+
+// ---- many rows: the (token, choice) pairs sorted by expert, products on the matrix cores -------
+#define MOE_TILE 64      // pairs per tile; an expert's pairs are padded up to whole tiles
+
+// One block.  order[pos] = the pair at sorted place pos (-1: padding), tile_expert[tile] = the
+// expert of the 64 places of a tile (-1: the tile is not used).  The place of a pair within its
+// expert's run depends on the order in which the threads arrive; nothing that is computed does.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int pairs,
+                                                        int experts, int* __restrict__ order,
+                                                        int* __restrict__ tile_expert, int max_tiles) {
+  __shared__ int s_count[MOE_MAX_EXPERTS];
+  __shared__ int s_start[MOE_MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) s_count[e] = 0;
+  for (int i = threadIdx.x; i < max_tiles * MOE_TILE; i += blockDim.x) order[i] = -1;
+  for (int i = threadIdx.x; i < max_tiles; i += blockDim.x) tile_expert[i] = -1;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&s_count[ids[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      s_start[e] = at;
+      at += (s_count[e] + MOE_TILE - 1) / MOE_TILE * MOE_TILE;
+    }
+    s_start[experts] = at;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+    for (int tile = s_start[e] / MOE_TILE; tile < s_start[e + 1] / MOE_TILE; ++tile) tile_expert[tile] = e;
+    s_count[e] = s_start[e];     // from here on: the next free place of the expert's run
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) order[atomicAdd(&s_count[ids[p]], 1)] = p;
+}
+
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float moe_f32x16;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
+#define MOE_LDS_STRIDE 80   // bytes between rows of a stage (64 bytes of k, padded)
+
+// A tile of 64 sorted pairs times 128 weight rows of the tile's expert, k in stages of 32.
+// HIDDEN: the weight rows are 64 gate rows and the 64 up rows of the same hidden columns, and
+// hidden[pair, column] = silu(gate) * up; the rows of A are the pairs' tokens (pair / top).
+// Otherwise: 128 output columns, out[pair, column] = weights[pair] * sum; the rows of A are the
+// pairs' hidden rows.  Four waves, 2 x 2: a wave has 32 pairs and two times 32 weight rows.
+template <bool HIDDEN>
+__global__ __launch_bounds__(256) void moe_grouped_kernel(
+    const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t expert_stride,
+    int w_rows, int k, const int* __restrict__ order, const int* __restrict__ tile_expert, int top,
+    const float* __restrict__ weights, bf16_t* __restrict__ hidden, float* __restrict__ out,
+    int64_t out_ld) {
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][(MOE_TILE + 128) * MOE_LDS_STRIDE];
+  __shared__ int s_pair[MOE_TILE];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int columns = HIDDEN ? w_rows / 2 : w_rows;      // output columns
+  const int n0 = blockIdx.y * (HIDDEN ? 64 : 128);
+  if (tid < MOE_TILE) s_pair[tid] = order[blockIdx.x * MOE_TILE + tid];
+  __syncthreads();
+  // staging: 16-byte chunks, 4 per row; A: 64 rows, one chunk a thread; W: 128 rows, two
+  const int chunk = (tid & 3) * 8;
+  const int a_row = tid >> 2;
+  const int a_pair = s_pair[a_row];
+  const bf16_t* a_src = a + (int64_t)(a_pair < 0 ? 0 : (HIDDEN ? a_pair / top : a_pair)) * lda + chunk;
+  const bf16_t* w_src[2];
+  bool w_ok[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int local = a_row + i * 64;      // 0..127
+    int row;
+    if (HIDDEN) row = (local < 64 ? 0 : columns) + n0 + (local & 63);
+    else row = n0 + local;
+    w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : row < w_rows;
+    w_src[i] = w + (int64_t)e * expert_stride + (int64_t)(w_ok[i] ? row : 0) * k + chunk;
+  }
+  uint4 stage_a, stage_w[2];
+  const uint4 zero = {0u, 0u, 0u, 0u};
+  auto load_global = [&](int k0) {
+    const bool k_ok = k0 + chunk < k;
+    const int kk = k_ok ? k0 : 0;
+    stage_a = *reinterpret_cast<const uint4*>(a_src + kk);
+    if (!(k_ok && a_pair >= 0)) stage_a = zero;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      stage_w[i] = *reinterpret_cast<const uint4*>(w_src[i] + kk);
+      if (!(k_ok && w_ok[i])) stage_w[i] = zero;
+    }
+  };
+  auto store_lds = [&](int buffer) {
+    const int offset = a_row * MOE_LDS_STRIDE + (tid & 3) * 16;
+    *reinterpret_cast<uint4*>(&lds[buffer][offset]) = stage_a;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      *reinterpret_cast<uint4*>(&lds[buffer][(MOE_TILE + i * 64) * MOE_LDS_STRIDE + offset]) = stage_w[i];
+  };
+  moe_f32x16 acc[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+  const int k_tiles = (k + 31) / 32;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    if (kt + 1 < k_tiles) load_global((kt + 1) * 32);
+    const unsigned char* stage = lds[kt & 1];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int kbyte = half * 32 + (lane >> 5) * 16;
+      const uint4 fa = *reinterpret_cast<const uint4*>(
+          &stage[(wave_m * 32 + (lane & 31)) * MOE_LDS_STRIDE + kbyte]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const uint4 fw = *reinterpret_cast<const uint4*>(
+            &stage[(MOE_TILE + j * 64 + wave_n * 32 + (lane & 31)) * MOE_LDS_STRIDE + kbyte]);
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const moe_bf16x8*>(&fa),
+                                                         *reinterpret_cast<const moe_bf16x8*>(&fw),
+                                                         acc[j], 0, 0, 0);
+      }
+    }
+    if (kt + 1 < k_tiles) store_lds((kt + 1) & 1);
+    __syncthreads();
+  }
+  // element i of an accumulator: row (i / 4) * 8 + (lane / 32) * 4 + i % 4, column lane % 32
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int pair = s_pair[wave_m * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)];
+    if (pair < 0) continue;
+    if (HIDDEN) {
+      const int col = n0 + wave_n * 32 + (lane & 31);
+      const float g = acc[0][i], u = acc[1][i];
+      if (col < columns) hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(g / (1.0f + expf(-g)) * u);
+    } else {
+      const float weight = weights[pair];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = n0 + j * 64 + wave_n * 32 + (lane & 31);
+        if (col < columns) out[(int64_t)pair * out_ld + col] = weight * acc[j][i];
+      }
+    }
+  }
+}
+
+// y[t, :] += sum_j out[t * top + j, :]
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ out,
+                                                          float* __restrict__ y, int width, int top) {
+  const int64_t t = blockIdx.x;
+  for (int d = threadIdx.x; d < width; d += 256) {
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) sum += out[(t * top + j) * width + d];
+    y[t * width + d] += sum;
+  }
+}
+
 extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2,
                               const int* ids, const float* weights, void* hidden, float* y,
                               int tokens, int width, int inner, int top, int dtype, void* stream) {
@@ -180,17 +455,57 @@ extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const
   constexpr int ROWS = 4;
   const dim3 grid1(tokens, (inner + 4 * ROWS - 1) / (4 * ROWS), top);
   const dim3 grid2(tokens, (width + 4 * ROWS - 1) / (4 * ROWS));
-  if (dtype == PS_F32) {
-    hipLaunchKernelGGL((moe_hidden_kernel<float, ROWS>), grid1, dim3(256), (size_t)width * 4, s,
-                       (const float*)x, x_ld, (const float*)w1, ids, (float*)hidden, width, inner);
-    hipLaunchKernelGGL((moe_down_kernel<float, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, s,
-                       (const float*)hidden, (const float*)w2, ids, weights, y, width, inner, top);
-  } else {
-    hipLaunchKernelGGL((moe_hidden_kernel<bf16_t, ROWS>), grid1, dim3(256), (size_t)width * 4, s,
-                       (const bf16_t*)x, x_ld, (const bf16_t*)w1, ids, (bf16_t*)hidden, width, inner);
-    hipLaunchKernelGGL((moe_down_kernel<bf16_t, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, s,
-                       (const bf16_t*)hidden, (const bf16_t*)w2, ids, weights, y, width, inner, top);
-  }
+  const bool wide1 = width % 8 == 0 && x_ld % 8 == 0, wide2 = inner % 8 == 0;
+#define PS_MOE_ROWS(T)                                                                             \
+  do {                                                                                             \
+    if (wide1)                                                                                     \
+      hipLaunchKernelGGL((moe_hidden_wide_kernel<T, ROWS>), grid1, dim3(256), (size_t)width * 4, s, \
+                         (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner);          \
+    else                                                                                           \
+      hipLaunchKernelGGL((moe_hidden_kernel<T, ROWS>), grid1, dim3(256), (size_t)width * 4, s,     \
+                         (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner);          \
+    if (wide2)                                                                                     \
+      hipLaunchKernelGGL((moe_down_wide_kernel<T, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, \
+                         s, (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top);   \
+    else                                                                                           \
+      hipLaunchKernelGGL((moe_down_kernel<T, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, s, \
+                         (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top);      \
+  } while (0)
+  if (dtype == PS_F32) PS_MOE_ROWS(float);
+  else PS_MOE_ROWS(bf16_t);
+#undef PS_MOE_ROWS
   PS_CHECK_LAUNCH("ps_moe_experts");
+  return 0;
+}
+
+extern "C" int ps_moe_grouped_tiles(int pairs, int experts) {
+  return (pairs + MOE_TILE - 1) / MOE_TILE + experts;
+}
+
+extern "C" int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w1, const void* w2,
+                                      const int* ids, const float* weights, void* hidden,
+                                      float* out, int* order, int* tile_expert, float* y,
+                                      int tokens, int width, int inner, int experts, int top,
+                                      void* stream) {
+  PS_REQUIRE(tokens >= 0 && width > 0 && inner > 0 && top > 0 && experts > 0 &&
+                 experts <= MOE_MAX_EXPERTS, "ps_moe_experts_grouped: bad sizes");
+  PS_REQUIRE(width % 8 == 0 && inner % 8 == 0 && x_ld % 8 == 0,
+             "ps_moe_experts_grouped: width %d and inner width %d must be multiples of 8", width, inner);
+  if (tokens == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int pairs = tokens * top;
+  const int tiles = ps_moe_grouped_tiles(pairs, experts);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, ids, pairs, experts, order, tile_expert,
+                     tiles);
+  hipLaunchKernelGGL(moe_grouped_kernel<true>, dim3(tiles, (inner + 63) / 64), dim3(256), 0, s,
+                     (const bf16_t*)x, x_ld, (const bf16_t*)w1, (int64_t)2 * inner * width, 2 * inner,
+                     width, order, tile_expert, top, weights, (bf16_t*)hidden, (float*)nullptr,
+                     (int64_t)0);
+  hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3(tiles, (width + 127) / 128), dim3(256), 0, s,
+                     (const bf16_t*)hidden, (int64_t)inner, (const bf16_t*)w2, (int64_t)width * inner,
+                     width, inner, order, tile_expert, top, weights, (bf16_t*)nullptr, out,
+                     (int64_t)width);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, s, out, y, width, top);
+  PS_CHECK_LAUNCH("ps_moe_experts_grouped");
   return 0;
 }

@@ -353,6 +353,15 @@ int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tokens, int wi
 int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2, const int* ids,
                    const float* weights, void* hidden, float* y, int tokens, int width, int inner,
                    int top, int dtype, void* stream);
+// The same for many rows in bfloat16 (width and inner multiples of 8): the (token, choice) pairs
+// are sorted by expert into tiles of 64 and multiplied on the matrix cores.  order:
+// [tiles * 64] int and tile_expert: [tiles] int scratch with tiles = ps_moe_grouped_tiles(tokens *
+// top, experts); out: [tokens * top, width] float scratch.
+int ps_moe_grouped_tiles(int pairs, int experts);
+int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w1, const void* w2, const int* ids,
+                           const float* weights, void* hidden, float* out, int* order,
+                           int* tile_expert, float* y, int tokens, int width, int inner, int experts,
+                           int top, void* stream);
 
 #ifdef __cplusplus
 }

@@ -62,6 +62,9 @@ _SIGNATURES = {
                          c_int, c_void_p],
     "ps_moe_route": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                      c_void_p, c_void_p, c_int, c_void_p],
+    "ps_moe_experts_grouped": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                               c_void_p],
     "ps_moe_experts": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                        c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_gla_output": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
@@ -1408,6 +1411,50 @@ def moe_route(x, router, groups, keep, top, scale, ids, weights):
     _call("ps_moe_route", x.data_ptr(), x.stride(0), router.data_ptr(), tokens, width, experts,
           int(groups), int(keep), int(top), float(scale), ids.data_ptr(), weights.data_ptr(),
           dtype_code(x.dtype), _stream())
+
+
+MOE_GROUPED_FROM = 128    # (token, choice) pairs from which the sorted path on the matrix cores is taken
+
+
+def moe_grouped_supported(dtype, width, inner) -> bool:
+    return dtype == torch.bfloat16 and width % 8 == 0 and inner % 8 == 0
+
+
+def moe_grouped_tiles(pairs, experts) -> int:
+    """Tiles of 64 sorted pairs that ``pairs`` pairs of ``experts`` experts can need at most."""
+    return -(-pairs // 64) + experts
+
+
+def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert, y):
+    """``moe_experts`` for many rows in bfloat16: the pairs sorted by expert, the products on the
+    matrix cores.  ``out``: float ``[>= tokens * top, width]``, ``order``: int32 ``[>= tiles * 64]``,
+    ``tile_expert``: int32 ``[>= tiles]`` scratch with ``tiles = moe_grouped_tiles(tokens * top, experts)``."""
+    _check(x, "x", torch.bfloat16, 2)
+    tokens, width = x.shape
+    _check(w1, "w1", x.dtype, 3)
+    _check(w2, "w2", x.dtype, 3)
+    experts, inner = w2.shape[0], w2.shape[2]
+    if (tuple(w1.shape) != (experts, 2 * inner, width) or tuple(w2.shape) != (experts, width, inner)
+            or not (w1.is_contiguous() and w2.is_contiguous()) or x.stride(1) != 1):
+        raise KernelError("moe_experts_grouped: w1 [experts, 2 * inner, width] and w2 [experts, width, inner] needed")
+    _check(ids, "ids", torch.int32, 2)
+    _check(weights, "weights", torch.float32, 2)
+    top = ids.shape[1]
+    if not (ids.is_contiguous() and weights.is_contiguous()) or weights.shape[1] != top:
+        raise KernelError("moe_experts_grouped: ids and weights must be contiguous [tokens, top]")
+    tiles = moe_grouped_tiles(tokens * top, experts)
+    _check(hidden, "hidden", x.dtype, 2)
+    if hidden.shape[0] < tokens * top or hidden.shape[1] != inner or not hidden.is_contiguous():
+        raise KernelError("moe_experts_grouped: hidden must be contiguous [>= tokens * top, inner]")
+    _float_rows(out, "out", tokens * top, width)
+    _check(order, "order", torch.int32, 1)
+    _check(tile_expert, "tile_expert", torch.int32, 1)
+    if order.numel() < tiles * 64 or tile_expert.numel() < tiles:
+        raise KernelError("moe_experts_grouped: the scratch for the sorted pairs is too small")
+    _float_rows(y, "y", tokens, width)
+    _call("ps_moe_experts_grouped", x.data_ptr(), x.stride(0), w1.data_ptr(), w2.data_ptr(), ids.data_ptr(),
+          weights.data_ptr(), hidden.data_ptr(), out.data_ptr(), order.data_ptr(), tile_expert.data_ptr(),
+          y.data_ptr(), tokens, width, inner, experts, top, _stream())
 
 
 def moe_experts(x, w1, w2, ids, weights, hidden, y):

@@ -157,6 +157,16 @@ class MixtureOfExperts(FeedForward):
         weights = workspace.first_rows("moe_weights", self.top, torch.float32, tokens)
         kernels.moe_route(x, self.router_weight, self.groups, self.keep, self.top, self.scale, ids,
                           weights)
-        hidden = workspace.rows("moe_hidden", self.inner, self.dtype,
-                                max_rows=workspace.max_rows * self.top)
-        kernels.moe_experts(x, self.gate_up_weight, self.down_weight, ids, weights, hidden, residual)
+        most = workspace.max_rows * self.top
+        hidden = workspace.rows("moe_hidden", self.inner, self.dtype, max_rows=most)
+        if (tokens * self.top >= kernels.MOE_GROUPED_FROM
+                and kernels.moe_grouped_supported(self.dtype, self.width, self.inner)):
+            # many rows: sorted by expert, tiles on the matrix cores
+            tiles = kernels.moe_grouped_tiles(most, self.experts)
+            kernels.moe_experts_grouped(
+                x, self.gate_up_weight, self.down_weight, ids, weights, hidden,
+                workspace.rows("moe_out", self.width, torch.float32, max_rows=most),
+                workspace.flat("moe_order", tiles * 64, torch.int32),
+                workspace.flat("moe_tiles", tiles, torch.int32), residual)
+        else:
+            kernels.moe_experts(x, self.gate_up_weight, self.down_weight, ids, weights, hidden, residual)

@@ -134,6 +134,55 @@ def test_experts_of_every_token(dtype, width, inner, experts, top):
     assert torch.allclose(y.double().cpu(), expected, atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("width,inner,experts,top,tokens", [(64, 40, 5, 2, 150), (128, 96, 4, 3, 70), (72, 136, 7, 1, 333),
+                                                            (256, 200, 3, 2, 64)])
+def test_experts_of_many_tokens_sorted_onto_the_matrix_cores(width, inner, experts, top, tokens):
+    """The path for many rows: pairs sorted by expert into tiles of 64 (experts with a few pairs,
+    with more than a tile, and one with none), against the plain sum and the path for few rows."""
+    kernels = _kernels()
+    g = torch.Generator().manual_seed(width + inner)
+    dtype = torch.bfloat16
+    x = torch.randn((tokens, width), generator=g).to(dtype)
+    w1 = (torch.randn((experts, 2 * inner, width), generator=g) / width ** 0.5).to(dtype)
+    w2 = (torch.randn((experts, width, inner), generator=g) / inner ** 0.5).to(dtype)
+    # the last expert gets nothing, the first most
+    ids = torch.stack([torch.randperm(experts - 1, generator=g)[:top] for _ in range(tokens)]).to(torch.int32)
+    ids[: tokens // 2, 0] = 0
+    for row in range(tokens // 2):
+        if top > 1 and int(ids[row, 1]) == 0:
+            ids[row, 1] = 1 if int(ids[row, min(2, top - 1)]) != 1 or top == 2 else experts - 2
+    weights = torch.rand((tokens, top), generator=g)
+    y0 = torch.randn((tokens, width), generator=g)
+    y = y0.clone().cuda()
+    pairs = tokens * top
+    tiles = kernels.moe_grouped_tiles(pairs, experts)
+    hidden = torch.empty((pairs, inner), dtype=dtype, device="cuda")
+    out = torch.empty((pairs, width), device="cuda")
+    order = torch.empty(tiles * 64, dtype=torch.int32, device="cuda")
+    tile_expert = torch.empty(tiles, dtype=torch.int32, device="cuda")
+    assert kernels.moe_grouped_supported(dtype, width, inner)
+    kernels.moe_experts_grouped(x.cuda(), w1.cuda(), w2.cuda(), ids.cuda(), weights.cuda(), hidden, out, order,
+                                tile_expert, y)
+    # every pair has one place, in a tile of its expert
+    placed = order.cpu()
+    assert sorted(placed[placed >= 0].tolist()) == list(range(pairs))
+    owners = tile_expert.cpu()
+    flat_ids = ids.reshape(-1)
+    for place in range(0, tiles * 64, 7):
+        if int(placed[place]) >= 0:
+            assert int(owners[place // 64]) == int(flat_ids[int(placed[place])])
+    rowwise = y0.clone().cuda()
+    kernels.moe_experts(x.cuda(), w1.cuda(), w2.cuda(), ids.cuda(), weights.cuda(), torch.empty_like(hidden), rowwise)
+    expected = y0.double().clone()
+    for t in range(0, tokens, 3):
+        for j in range(top):
+            e = int(ids[t, j])
+            expected[t] += float(weights[t, j]) * plain.gated(
+                x[t:t + 1].double(), w1[e, :inner].double(), w1[e, inner:].double(), w2[e].double())[0]
+    assert torch.allclose(y.double().cpu()[::3], expected[::3], atol=3e-2, rtol=3e-2)
+    assert torch.allclose(y, rowwise, atol=2e-2, rtol=2e-2)
+
+
 def _scan_inputs(g, total, channels, states, rank):
     proj = torch.randn((total, 2 * channels + 3), generator=g)
     low = torch.randn((total, rank + 2 * states + 2), generator=g)
