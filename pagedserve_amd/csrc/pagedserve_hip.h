@@ -322,11 +322,15 @@ int ps_step_size(const float* low, int64_t ld, int rank, const void* w, const fl
 // Per item and channel, token after token: S[n] = exp(dt A[n]) S[n] + dt x B_t[n] with
 // A = -exp(a_log[c, n]); y = (sum_n S[n] C_t[n] + skip[c] x) * silu(z) with z = proj[:, z_col + c].
 // B and C: bc[t * bc_ld + b_col / c_col + n].  Writes the states and the last raw inputs back.
+// records / sums (or null for both): scratch of (pieces + items) * channels * states and
+// (pieces + items) * channels floats with pieces = ps_selective_pieces(tokens, items); with them
+// the items are cut into pieces that run side by side (for steps with long portions).
+int ps_selective_pieces(int tokens, int items);
 int ps_selective_scan(const void* x, const float* dt, const float* bc, int64_t bc_ld, int b_col,
                       int c_col, const float* proj, int64_t ld, int u_col, int z_col,
                       const float* a_log, const float* skip, float* state, void* y,
                       const int* cu_tokens, const int* slots, int items, int channels, int states,
-                      int taps, int dtype, void* stream);
+                      int taps, int tokens, float* records, float* sums, int dtype, void* stream);
 
 // ---- a stream whose sublayers add into a scratch row ------------------------------------------
 // h += factor * y + bias (y, bias: null for none); zero[...] = 0 (may be y); if gamma:

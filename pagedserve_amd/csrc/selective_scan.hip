@@ -62,85 +62,225 @@ __global__ __launch_bounds__(256) void step_size_kernel(
   }
 }
 
-// The recurrence.  A block of one wave owns 64 / LPC channels of one item and walks the item's
-// tokens in order; a channel's states are dealt to LPC neighbouring lanes (state n to lane
-// n % LPC), SPL to a lane, in registers.  B and C of SS_CHUNK tokens wait in LDS.  At the end
-// the states and the last taps - 1 raw inputs go back to the slot.
+// The recurrence.  A block of one wave owns 64 / LPC channels of one item and walks tokens in
+// order; a channel's states are dealt to LPC neighbouring lanes (state n to lane n % LPC), SPL to a
+// lane, in registers.  B and C of SS_CHUNK tokens wait in LDS.
 #define SS_CHUNK 16
+struct ScanArgs {
+  const float* dt;
+  const float* bc;
+  int64_t bc_ld;
+  int b_col, c_col;
+  const float* proj;
+  int64_t ld;
+  int u_col, z_col;
+  const float* a_log;
+  const float* skip;
+  float* state;
+  const int* cu_tokens;
+  const int* slots;
+  int channels, states, taps;
+};
+
+// Tokens first .. last - 1 of one item for the block's channels, from the states in S.  EMIT:
+// the outputs are written; else only the states move, and the lanes get the sum of the step sizes.
+template <typename T, int LPC, int SPL, bool EMIT>
+__device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T* __restrict__ y,
+                                   int first, int last, int c, int cc, bool live, float (&S)[SPL],
+                                   const float (&A)[SPL], float* s_bc) {
+  const int lane = threadIdx.x;
+  const int part = lane % LPC;
+  const int states = p.states, channels = p.channels;
+  const float d_skip = EMIT ? p.skip[cc] : 0.f;
+  float steps = 0.f;
+  for (int base = first; base < last; base += SS_CHUNK) {
+    const int count = (last - base) < SS_CHUNK ? (last - base) : SS_CHUNK;
+    __syncthreads();
+    for (int idx = lane; idx < count * 2 * states; idx += 64) {
+      const int tt = idx / (2 * states);
+      const int n = idx - tt * 2 * states;
+      s_bc[idx] = p.bc[(int64_t)(base + tt) * p.bc_ld + (n < states ? p.b_col + n : p.c_col + n - states)];
+    }
+    __syncthreads();
+    for (int tt = 0; tt < count; ++tt) {
+      const int64_t t = base + tt;
+      const float step = p.dt[t * channels + cc];
+      const float xv = to_float<T>(x[t * channels + cc]);
+      const float* b_row = s_bc + tt * 2 * states;
+      const float* c_row = b_row + states;
+      const float sx = step * xv;
+      float sum = 0.f;
+      steps += step;
+#pragma unroll
+      for (int i = 0; i < SPL; ++i) {
+        const int n = part + i * LPC;
+        if (n < states) {
+          S[i] = fmaf(expf(step * A[i]), S[i], sx * b_row[n]);
+          if (EMIT) sum = fmaf(S[i], c_row[n], sum);
+        }
+      }
+      if (EMIT) {
+        sum = lanes_sum<LPC>(sum);
+        if (part == 0 && live) {
+          const float z = p.proj[t * p.ld + p.z_col + c];
+          y[t * channels + c] = from_float<T>(fmaf(d_skip, xv, sum) * silu_f(z));
+        }
+      }
+    }
+  }
+  return steps;
+}
+
+// The slot's last taps - 1 raw inputs of (what it kept, then tokens t0 .. t1 - 1), oldest first.
+__device__ inline void keep_inputs(const ScanArgs& p, float* kept, int t0, int t1, int c) {
+  const int count = t1 - t0;
+  for (int j = 0; j < p.taps - 1; ++j) {
+    const int local = count - (p.taps - 1) + j;      // place among this step's tokens
+    // (ascending j reads kept[j + count] with count >= 1: never a place already written)
+    kept[j] = local >= 0 ? p.proj[(int64_t)(t0 + local) * p.ld + p.u_col + c] : kept[j + count];
+  }
+}
+
+// One block walks all tokens of its item: the shape for decoded tokens and short portions.
 template <typename T, int LPC, int SPL>
-__global__ __launch_bounds__(64) void selective_scan_kernel(
-    const T* __restrict__ x, const float* __restrict__ dt, const float* __restrict__ bc, int64_t bc_ld,
-    int b_col, int c_col, const float* __restrict__ proj, int64_t ld, int u_col, int z_col,
-    const float* __restrict__ a_log, const float* __restrict__ skip, float* __restrict__ state,
-    T* __restrict__ y, const int* __restrict__ cu_tokens, const int* __restrict__ slots,
-    int channels, int states, int taps) {
+__global__ __launch_bounds__(64) void selective_scan_kernel(ScanArgs p, const T* __restrict__ x,
+                                                            T* __restrict__ y) {
   constexpr int CPB = 64 / LPC;
   extern __shared__ float s_bc[];            // [SS_CHUNK][2 * states]
   const int item = blockIdx.x;
   const int lane = threadIdx.x;
   const int part = lane % LPC;
   const int c = blockIdx.y * CPB + lane / LPC;
-  const bool live = c < channels;
-  const int cc = live ? c : channels - 1;
-  const int t0 = cu_tokens[item], t1 = cu_tokens[item + 1];
-  const int row = states + taps - 1;
-  float* mine = state + ((int64_t)slots[item] * channels + cc) * row;
+  const bool live = c < p.channels;
+  const int cc = live ? c : p.channels - 1;
+  const int t0 = p.cu_tokens[item], t1 = p.cu_tokens[item + 1];
+  const int row = p.states + p.taps - 1;
+  float* mine = p.state + ((int64_t)p.slots[item] * p.channels + cc) * row;
   float S[SPL], A[SPL];
 #pragma unroll
   for (int i = 0; i < SPL; ++i) {
     const int n = part + i * LPC;
-    S[i] = n < states ? mine[n] : 0.f;
-    A[i] = n < states ? -expf(a_log[(int64_t)cc * states + n]) : 0.f;
+    S[i] = n < p.states ? mine[n] : 0.f;
+    A[i] = n < p.states ? -expf(p.a_log[(int64_t)cc * p.states + n]) : 0.f;
   }
-  const float d_skip = skip[cc];
-  for (int base = t0; base < t1; base += SS_CHUNK) {
-    const int count = (t1 - base) < SS_CHUNK ? (t1 - base) : SS_CHUNK;
-    __syncthreads();
-    for (int idx = lane; idx < count * 2 * states; idx += 64) {
-      const int tt = idx / (2 * states);
-      const int n = idx - tt * 2 * states;
-      s_bc[idx] = bc[(int64_t)(base + tt) * bc_ld + (n < states ? b_col + n : c_col + n - states)];
-    }
-    __syncthreads();
-    for (int tt = 0; tt < count; ++tt) {
-      const int64_t t = base + tt;
-      const float step = dt[t * channels + cc];
-      const float xv = to_float<T>(x[t * channels + cc]);
-      const float* b_row = s_bc + tt * 2 * states;
-      const float* c_row = b_row + states;
-      const float sx = step * xv;
-      float sum = 0.f;
-#pragma unroll
-      for (int i = 0; i < SPL; ++i) {
-        const int n = part + i * LPC;
-        if (n < states) {
-          S[i] = fmaf(expf(step * A[i]), S[i], sx * b_row[n]);
-          sum = fmaf(S[i], c_row[n], sum);
-        }
-      }
-      sum = lanes_sum<LPC>(sum);
-      if (part == 0 && live) {
-        const float z = proj[t * ld + z_col + c];
-        y[t * channels + c] = from_float<T>(fmaf(d_skip, xv, sum) * silu_f(z));
-      }
-    }
-  }
+  scan_range<T, LPC, SPL, true>(p, x, y, t0, t1, c, cc, live, S, A, s_bc);
   if (!live) return;
 #pragma unroll
   for (int i = 0; i < SPL; ++i) {
     const int n = part + i * LPC;
-    if (n < states) mine[n] = S[i];
+    if (n < p.states) mine[n] = S[i];
   }
-  if (part == 0 && t1 > t0) {
-    // the last taps - 1 raw inputs of (what the slot kept, then this step's), oldest first
-    const int count = t1 - t0;
-    float* kept = mine + states;
-    for (int j = 0; j < taps - 1; ++j) {
-      const int local = count - (taps - 1) + j;      // place among this step's tokens
-      // (ascending j reads kept[j + count] with count >= 1: never a place already written)
-      kept[j] = local >= 0 ? proj[(int64_t)(t0 + local) * ld + u_col + c] : kept[j + count];
+  if (part == 0 && t1 > t0) keep_inputs(p, mine + p.states, t0, t1, c);
+}
+
+// Long portions are cut into pieces of SS_PIECE tokens that run side by side.  The recurrence
+// is linear in the state, S_end = P S_start + E with P = exp(A * sum of the piece's step sizes)
+// and E what the piece leaves from a zero state, so three launches do it:
+//   1. every piece from zero: E and the sum of its step sizes (the first piece of an item also
+//      copies the slot's state aside);
+//   2. per item, piece after piece: the state at each piece's start, and the item's last state
+//      into the slot;
+//   3. every piece again from its true start, now writing the outputs.
+// Records: [entry][channels][states] floats and [entry][channels] sums, an item's entries one
+// behind the other: its start, then its pieces.
+#define SS_PIECE 32
+struct PieceOf {
+  int item, piece, pieces, entry;     // entry: the record of the item's start
+};
+
+// The (item, piece) of the block's place among all pieces of the step; item < 0: none.
+__device__ inline PieceOf find_piece(const int* cu_tokens, int items, int place) {
+  PieceOf found = {-1, 0, 0, 0};
+  int entry = 0;
+  for (int i = 0; i < items; ++i) {
+    const int pieces = (cu_tokens[i + 1] - cu_tokens[i] + SS_PIECE - 1) / SS_PIECE;
+    if (place < pieces) {
+      found.item = i;
+      found.piece = place;
+      found.pieces = pieces;
+      found.entry = entry;
+      return found;
+    }
+    place -= pieces;
+    entry += pieces + 1;
+  }
+  return found;
+}
+
+template <typename T, int LPC, int SPL, bool EMIT>
+__global__ __launch_bounds__(64) void selective_pieces_kernel(ScanArgs p, const T* __restrict__ x,
+                                                              T* __restrict__ y, int items,
+                                                              float* __restrict__ records,
+                                                              float* __restrict__ sums) {
+  constexpr int CPB = 64 / LPC;
+  extern __shared__ float s_bc[];
+  const PieceOf at = find_piece(p.cu_tokens, items, blockIdx.x);
+  if (at.item < 0) return;
+  const int lane = threadIdx.x;
+  const int part = lane % LPC;
+  const int c = blockIdx.y * CPB + lane / LPC;
+  const bool live = c < p.channels;
+  const int cc = live ? c : p.channels - 1;
+  const int t0 = p.cu_tokens[at.item], t1 = p.cu_tokens[at.item + 1];
+  const int first = t0 + at.piece * SS_PIECE;
+  const int last = first + SS_PIECE < t1 ? first + SS_PIECE : t1;
+  const int64_t per_entry = (int64_t)p.channels * p.states;
+  float* record = records + (at.entry + 1 + at.piece) * per_entry + (int64_t)cc * p.states;
+  const int row = p.states + p.taps - 1;
+  float* mine = p.state + ((int64_t)p.slots[at.item] * p.channels + cc) * row;
+  float S[SPL], A[SPL];
+#pragma unroll
+  for (int i = 0; i < SPL; ++i) {
+    const int n = part + i * LPC;
+    A[i] = n < p.states ? -expf(p.a_log[(int64_t)cc * p.states + n]) : 0.f;
+    S[i] = (EMIT && n < p.states) ? record[n] : 0.f;
+  }
+  if (!EMIT && at.piece == 0 && live) {
+    float* start = records + at.entry * per_entry + (int64_t)cc * p.states;
+#pragma unroll
+    for (int i = 0; i < SPL; ++i) {
+      const int n = part + i * LPC;
+      if (n < p.states) start[n] = mine[n];
     }
   }
+  const float steps = scan_range<T, LPC, SPL, EMIT>(p, x, y, first, last, c, cc, live, S, A, s_bc);
+  if (!live) return;
+  if (!EMIT) {
+#pragma unroll
+    for (int i = 0; i < SPL; ++i) {
+      const int n = part + i * LPC;
+      if (n < p.states) record[n] = S[i];
+    }
+    if (part == 0) sums[(int64_t)(at.entry + 1 + at.piece) * p.channels + c] = steps;
+  } else if (at.piece == at.pieces - 1 && part == 0) {
+    keep_inputs(p, mine + p.states, t0, t1, c);
+  }
+}
+
+// Launch 2: a thread per (channel, state) of an item.
+__global__ __launch_bounds__(256) void selective_join_kernel(ScanArgs p, float* __restrict__ records,
+                                                             const float* __restrict__ sums) {
+  const int item = blockIdx.x;
+  const int64_t per_entry = (int64_t)p.channels * p.states;
+  const int64_t index = (int64_t)blockIdx.y * 256 + threadIdx.x;
+  if (index >= per_entry) return;
+  int entry = 0;
+  for (int i = 0; i < item; ++i)
+    entry += (p.cu_tokens[i + 1] - p.cu_tokens[i] + SS_PIECE - 1) / SS_PIECE + 1;
+  const int pieces = (p.cu_tokens[item + 1] - p.cu_tokens[item] + SS_PIECE - 1) / SS_PIECE;
+  if (pieces == 0) return;
+  const int c = (int)(index / p.states), n = (int)(index - (int64_t)c * p.states);
+  const float a = -expf(p.a_log[index]);
+  float s = records[entry * per_entry + index];
+  for (int j = 0; j < pieces; ++j) {
+    float* record = records + (entry + 1 + j) * per_entry + index;
+    const float left = *record;
+    const float decay = expf(a * sums[(int64_t)(entry + 1 + j) * p.channels + c]);
+    *record = s;
+    s = fmaf(decay, s, left);
+  }
+  const int row = p.states + p.taps - 1;
+  p.state[((int64_t)p.slots[item] * p.channels + c) * row + n] = s;
 }
 
 extern "C" int ps_conv_silu(const float* proj, int64_t ld, int u_col, const float* w,
@@ -181,22 +321,44 @@ extern "C" int ps_step_size(const float* low, int64_t ld, int rank, const void* 
   return 0;
 }
 
+extern "C" int ps_selective_pieces(int tokens, int items) {
+  return tokens / SS_PIECE + items;      // no step of that many tokens and items has more pieces
+}
+
+// records / sums: scratch for the launch in pieces, [(pieces + items) * channels * states] and
+// [(pieces + items) * channels] floats with pieces = ps_selective_pieces(tokens, items); null:
+// every item is walked by one block.
 extern "C" int ps_selective_scan(const void* x, const float* dt, const float* bc, int64_t bc_ld,
                                  int b_col, int c_col, const float* proj, int64_t ld, int u_col,
                                  int z_col, const float* a_log, const float* skip, float* state,
                                  void* y, const int* cu_tokens, const int* slots, int items,
-                                 int channels, int states, int taps, int dtype, void* stream) {
+                                 int channels, int states, int taps, int tokens, float* records,
+                                 float* sums, int dtype, void* stream) {
   PS_REQUIRE(items >= 0 && channels > 0 && states > 0 && taps >= 1, "ps_selective_scan: bad sizes");
   PS_REQUIRE(states <= 256, "ps_selective_scan: %d states per channel, at most 256", states);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_selective_scan: unknown dtype %d", dtype);
+  PS_REQUIRE((records == nullptr) == (sums == nullptr), "ps_selective_scan: records and sums go together");
   if (items == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const size_t lds = (size_t)SS_CHUNK * 2 * states * sizeof(float);
+  const ScanArgs p = {dt, bc, bc_ld, b_col, c_col, proj, ld, u_col, z_col, a_log, skip, state,
+                      cu_tokens, slots, channels, states, taps};
+  const int pieces = ps_selective_pieces(tokens, items);
 #define PS_LAUNCH_SS_T(T, LPC, SPL)                                                               \
-  hipLaunchKernelGGL((selective_scan_kernel<T, LPC, SPL>),                                        \
-                     dim3(items, (channels + 64 / LPC - 1) / (64 / LPC)), dim3(64), lds, s,       \
-                     (const T*)x, dt, bc, bc_ld, b_col, c_col, proj, ld, u_col, z_col, a_log, skip, \
-                     state, (T*)y, cu_tokens, slots, channels, states, taps)
+  do {                                                                                            \
+    const int blocks = (channels + 64 / LPC - 1) / (64 / LPC);                                    \
+    if (records == nullptr) {                                                                     \
+      hipLaunchKernelGGL((selective_scan_kernel<T, LPC, SPL>), dim3(items, blocks), dim3(64), lds, s, \
+                         p, (const T*)x, (T*)y);                                                  \
+    } else {                                                                                      \
+      hipLaunchKernelGGL((selective_pieces_kernel<T, LPC, SPL, false>), dim3(pieces, blocks),     \
+                         dim3(64), lds, s, p, (const T*)x, (T*)y, items, records, sums);          \
+      hipLaunchKernelGGL(selective_join_kernel, dim3(items, (channels * states + 255) / 256),     \
+                         dim3(256), 0, s, p, records, sums);                                      \
+      hipLaunchKernelGGL((selective_pieces_kernel<T, LPC, SPL, true>), dim3(pieces, blocks),      \
+                         dim3(64), lds, s, p, (const T*)x, (T*)y, items, records, sums);          \
+    }                                                                                             \
+  } while (0)
 #define PS_LAUNCH_SS(LPC, SPL)                  \
   do {                                          \
     if (dtype == PS_F32) {                      \

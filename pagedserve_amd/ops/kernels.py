@@ -54,7 +54,7 @@ _SIGNATURES = {
                      c_void_p],
     "ps_selective_scan": [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                           c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "ps_stream_step": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
                        c_int, c_int, c_int, c_void_p],
     "ps_silu_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
@@ -1316,10 +1316,22 @@ def step_size(low, w, bias, dt):
           tokens, channels, dtype_code(w.dtype), _stream())
 
 
+SCAN_PIECE = 32     # tokens of a piece of the selective scan's launch in pieces
+
+
+def selective_scan_records(tokens, items, channels, states):
+    """Floats of the two scratch buffers (records, sums) that ``selective_scan`` needs to cut a
+    step of so many tokens and items into pieces."""
+    entries = tokens // SCAN_PIECE + 2 * items
+    return entries * channels * states, entries * channels
+
+
 def selective_scan(x, dt, bc, b_col, c_col, proj, u_col, z_col, a_log, skip, state, y, cu_tokens,
-                   slots, taps):
+                   slots, taps, scratch=None):
     """The selective recurrence over the step's items (``csrc/pagedserve_hip.h: ps_selective_scan``);
-    ``state``: float ``[slots, channels, states + taps - 1]``."""
+    ``state``: float ``[slots, channels, states + taps - 1]``.  ``scratch = (records, sums)``: float
+    buffers of at least ``selective_scan_records(...)`` elements; with them the items are cut into
+    pieces that run side by side (three launches: for steps with long portions)."""
     _check(x, "x", ndim=2)
     tokens, channels = x.shape
     _check(a_log, "a_log", torch.float32, 2)
@@ -1339,10 +1351,18 @@ def selective_scan(x, dt, bc, b_col, c_col, proj, u_col, z_col, a_log, skip, sta
     if y.shape[0] < tokens or y.shape[1] != channels or not y.is_contiguous():
         raise KernelError("selective_scan: y must be contiguous [>= tokens, channels]")
     items = _step_items(cu_tokens, slots, "selective_scan")
+    records = sums = None
+    if scratch is not None:
+        records, sums = scratch
+        need = selective_scan_records(tokens, items, channels, states)
+        _check(records, "records", torch.float32, 1)
+        _check(sums, "sums", torch.float32, 1)
+        if records.numel() < need[0] or sums.numel() < need[1]:
+            raise KernelError("selective_scan: the scratch for the pieces is too small")
     _call("ps_selective_scan", x.data_ptr(), dt.data_ptr(), bc.data_ptr(), bc.stride(0), b_col, c_col,
           proj.data_ptr(), proj.stride(0), u_col, z_col, a_log.data_ptr(), skip.data_ptr(),
           state.data_ptr(), y.data_ptr(), cu_tokens.data_ptr(), slots.data_ptr(), items, channels,
-          states, taps, dtype_code(x.dtype), _stream())
+          states, taps, tokens, _ptr(records), _ptr(sums), dtype_code(x.dtype), _stream())
 
 
 def stream_step(h, tokens, width, add=None, bias=None, norm=None, zero=None):

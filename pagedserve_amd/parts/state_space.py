@@ -28,6 +28,9 @@ class SelectiveScan(Mixer):
 
     accepts_pending_norm = True
 
+    # tokens beyond one per item from which a step's items are cut into pieces that run side by side
+    PIECES_FROM = 96
+
     def __init__(self, width: int, dtype, inner: int, states: int, dt_rank: int, taps: int):
         if not 0 < states <= 256:
             raise ValueError(f"states {states} must lie in 1..256")
@@ -82,8 +85,17 @@ class SelectiveScan(Mixer):
         dt = workspace.first_rows("scan_dt", inner, torch.float32, tokens)
         kernels.step_size(low[:, :rank], self.dt_weight, self.dt_bias, dt)
         y = workspace.first_rows("scan_y", inner, self.dtype, tokens)
+        scratch = None
+        items = ctx.slots.numel()
+        if tokens - items >= self.PIECES_FROM:
+            # some item brings a long portion: pieces of it run side by side.  The scratch is
+            # asked for at its largest, so that it never moves under recorded launches.
+            most = kernels.selective_scan_records(workspace.max_rows, cache.state.shape[0], inner, states)
+            scratch = (workspace.flat("scan_records", most[0], torch.float32),
+                       workspace.flat("scan_sums", most[1], torch.float32))
         kernels.selective_scan(activated, dt, low, rank, rank + states, proj, 0, inner, self.a_log,
-                               self.skip, cache.state, y, ctx.cu_tokens, ctx.slots, self.taps)
+                               self.skip, cache.state, y, ctx.cu_tokens, ctx.slots, self.taps,
+                               scratch=scratch)
         kernels.linear(y, self.out_weight, None, residual, epilogue="residual",
                        packed=self.out_packed, memo=site_memo(self._memo_out, workspace),
                        shared=ctx.shared_calls)
