@@ -83,6 +83,69 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
   }
 }
 
+// The same for up to 64 experts: a block of four waves per token, the waves share the experts'
+// logits between them, and the choice is made with an expert per lane.  Ties go to the
+// expert (and the group) with the lower number, as above.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_wave_kernel(
+    const T* __restrict__ x, int64_t x_ld, const float* __restrict__ w, int width, int experts,
+    int groups, int keep, int top, float scale, int* __restrict__ ids, float* __restrict__ weights) {
+  __shared__ float s_score[64];
+  __shared__ float s_group[64];
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const T* row = x + t * x_ld;
+  for (int e = wave; e < experts; e += 4) {
+    const float* w_row = w + (int64_t)e * width;
+    float sum = 0.f;
+    for (int d = lane; d < width; d += 64) sum = fmaf(to_float<T>(row[d]), w_row[d], sum);
+    sum = wave_sum(sum);
+    if (lane == 0) s_score[e] = sum;
+  }
+  __syncthreads();
+  // (all four waves choose, from the same numbers; the first one writes)
+  const bool mine = lane < experts;
+  const float z = mine ? s_score[lane] : -INFINITY;
+  __syncthreads();
+  const float p = mine ? expf(z - wave_max(z)) : 0.f;
+  const float score = p / wave_sum(p);
+  bool open = mine;
+  if (groups > 1 && keep < groups) {
+    const int size = experts / groups;
+    s_score[lane] = score;
+    __syncthreads();
+    if (lane < groups) {
+      float best = -INFINITY;
+      for (int e = lane * size; e < (lane + 1) * size; ++e) best = fmaxf(best, s_score[e]);
+      s_group[lane] = best;
+    }
+    __syncthreads();
+    if (mine) {
+      const int g = lane / size;
+      const float own = s_group[g];
+      int ahead = 0;
+      for (int other = 0; other < groups; ++other) {
+        const float theirs = s_group[other];
+        ahead += (theirs > own || (theirs == own && other < g)) ? 1 : 0;
+      }
+      open = ahead < keep;
+    }
+  }
+  for (int j = 0; j < top; ++j) {
+    const float offer = open ? score : -1.f;
+    const float best = wave_max(offer);
+    const unsigned long long holders = __ballot(offer == best);
+    const int chosen = holders ? __builtin_ctzll(holders) : 0;
+    if (lane == chosen) {
+      open = false;
+      if (wave == 0) {
+        ids[t * top + j] = chosen;
+        weights[t * top + j] = (best < 0.f ? 0.f : best) * scale;
+      }
+    }
+  }
+}
+
 // hidden[(t, j), c] = silu(W_gate,e[c] . x_t) * (W_up,e[c] . x_t) for e = ids[t, j].  The
 // experts' first matrices lie one behind the other, [experts][gate rows | up rows][width].
 // A block of four waves per (token, choice) and 4 * ROWS hidden columns; the lanes share a dot
@@ -157,7 +220,14 @@ extern "C" int ps_moe_route(const void* x, int64_t x_ld, const float* w, int tok
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_moe_route: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == PS_F32)
+  if (experts <= 64) {
+    if (dtype == PS_F32)
+      hipLaunchKernelGGL(moe_route_wave_kernel<float>, dim3(tokens), dim3(256), 0, s, (const float*)x,
+                         x_ld, w, width, experts, groups, keep, top, scale, ids, weights);
+    else
+      hipLaunchKernelGGL(moe_route_wave_kernel<bf16_t>, dim3(tokens), dim3(256), 0, s, (const bf16_t*)x,
+                         x_ld, w, width, experts, groups, keep, top, scale, ids, weights);
+  } else if (dtype == PS_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, dim3(tokens), dim3(64), 0, s, (const float*)x, x_ld, w,
                        width, experts, groups, keep, top, scale, ids, weights);
   else
@@ -287,10 +357,10 @@ __global__ __launch_bounds__(256) void moe_down_wide_kernel(
 }
 
 // ---- many rows: the (token, choice) pairs sorted by expert, products on the matrix cores -------
-#define MOE_TILE 64      // pairs per tile; an expert's pairs are padded up to whole tiles
+#define MOE_TILE 128     // pairs per tile; an expert's pairs are padded up to whole tiles
 
 // One block.  order[pos] = the pair at sorted place pos (-1: padding), tile_expert[tile] = the
-// expert of the 64 places of a tile (-1: the tile is not used).  The place of a pair within its
+// expert of the MOE_TILE places of a tile (-1: the tile is not used).  The place of a pair within its
 // expert's run depends on the order in which the threads arrive; nothing that is computed does.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int pairs,
                                                         int experts, int* __restrict__ order,
@@ -324,11 +394,11 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float moe_f32x16;
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
 #define MOE_LDS_STRIDE 80   // bytes between rows of a stage (64 bytes of k, padded)
 
-// A tile of 64 sorted pairs times 128 weight rows of the tile's expert, k in stages of 32.
+// A tile of 128 sorted pairs times 128 weight rows of the tile's expert, k in stages of 32.
 // HIDDEN: the weight rows are 64 gate rows and the 64 up rows of the same hidden columns, and
 // hidden[pair, column] = silu(gate) * up; the rows of A are the pairs' tokens (pair / top).
 // Otherwise: 128 output columns, out[pair, column] = weights[pair] * sum; the rows of A are the
-// pairs' hidden rows.  Four waves, 2 x 2: a wave has 32 pairs and two times 32 weight rows.
+// pairs' hidden rows.  Four waves, 2 x 2: a wave has 64 pairs and two times 32 weight rows.
 template <bool HIDDEN>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t expert_stride,
@@ -346,15 +416,18 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   const int n0 = blockIdx.y * (HIDDEN ? 64 : 128);
   if (tid < MOE_TILE) s_pair[tid] = order[blockIdx.x * MOE_TILE + tid];
   __syncthreads();
-  // staging: 16-byte chunks, 4 per row; A: 64 rows, one chunk a thread; W: 128 rows, two
+  // staging: 16-byte chunks, 4 per row; A and W: 128 rows each, two chunks a thread
   const int chunk = (tid & 3) * 8;
   const int a_row = tid >> 2;
-  const int a_pair = s_pair[a_row];
-  const bf16_t* a_src = a + (int64_t)(a_pair < 0 ? 0 : (HIDDEN ? a_pair / top : a_pair)) * lda + chunk;
+  const bf16_t* a_src[2];
+  bool a_ok[2];
   const bf16_t* w_src[2];
   bool w_ok[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
+    const int a_pair = s_pair[a_row + i * 64];
+    a_ok[i] = a_pair >= 0;
+    a_src[i] = a + (int64_t)(a_pair < 0 ? 0 : (HIDDEN ? a_pair / top : a_pair)) * lda + chunk;
     const int local = a_row + i * 64;      // 0..127
     int row;
     if (HIDDEN) row = (local < 64 ? 0 : columns) + n0 + (local & 63);
@@ -362,31 +435,34 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : row < w_rows;
     w_src[i] = w + (int64_t)e * expert_stride + (int64_t)(w_ok[i] ? row : 0) * k + chunk;
   }
-  uint4 stage_a, stage_w[2];
+  uint4 stage_a[2], stage_w[2];
   const uint4 zero = {0u, 0u, 0u, 0u};
   auto load_global = [&](int k0) {
     const bool k_ok = k0 + chunk < k;
     const int kk = k_ok ? k0 : 0;
-    stage_a = *reinterpret_cast<const uint4*>(a_src + kk);
-    if (!(k_ok && a_pair >= 0)) stage_a = zero;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
+      stage_a[i] = *reinterpret_cast<const uint4*>(a_src[i] + kk);
+      if (!(k_ok && a_ok[i])) stage_a[i] = zero;
       stage_w[i] = *reinterpret_cast<const uint4*>(w_src[i] + kk);
       if (!(k_ok && w_ok[i])) stage_w[i] = zero;
     }
   };
   auto store_lds = [&](int buffer) {
     const int offset = a_row * MOE_LDS_STRIDE + (tid & 3) * 16;
-    *reinterpret_cast<uint4*>(&lds[buffer][offset]) = stage_a;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i) {
+      *reinterpret_cast<uint4*>(&lds[buffer][i * 64 * MOE_LDS_STRIDE + offset]) = stage_a[i];
       *reinterpret_cast<uint4*>(&lds[buffer][(MOE_TILE + i * 64) * MOE_LDS_STRIDE + offset]) = stage_w[i];
+    }
   };
-  moe_f32x16 acc[2];
+  moe_f32x16 acc[2][2];      // [rows of 32 pairs][weight rows]
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int r = 0; r < 2; ++r)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[r][j][i] = 0.f;
   const int k_tiles = (k + 31) / 32;
   load_global(0);
   store_lds(0);
@@ -397,35 +473,42 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int kbyte = half * 32 + (lane >> 5) * 16;
-      const uint4 fa = *reinterpret_cast<const uint4*>(
-          &stage[(wave_m * 32 + (lane & 31)) * MOE_LDS_STRIDE + kbyte]);
+      uint4 fa[2], fw[2];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const uint4 fw = *reinterpret_cast<const uint4*>(
+      for (int r = 0; r < 2; ++r)
+        fa[r] = *reinterpret_cast<const uint4*>(
+            &stage[(wave_m * 64 + r * 32 + (lane & 31)) * MOE_LDS_STRIDE + kbyte]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        fw[j] = *reinterpret_cast<const uint4*>(
             &stage[(MOE_TILE + j * 64 + wave_n * 32 + (lane & 31)) * MOE_LDS_STRIDE + kbyte]);
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const moe_bf16x8*>(&fa),
-                                                         *reinterpret_cast<const moe_bf16x8*>(&fw),
-                                                         acc[j], 0, 0, 0);
-      }
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[r][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              *reinterpret_cast<const moe_bf16x8*>(&fa[r]), *reinterpret_cast<const moe_bf16x8*>(&fw[j]),
+              acc[r][j], 0, 0, 0);
     }
     if (kt + 1 < k_tiles) store_lds((kt + 1) & 1);
     __syncthreads();
   }
   // element i of an accumulator: row (i / 4) * 8 + (lane / 32) * 4 + i % 4, column lane % 32
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int pair = s_pair[wave_m * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)];
+  for (int ri = 0; ri < 32; ++ri) {
+    const int r = ri >> 4, i = ri & 15;
+    const int pair = s_pair[wave_m * 64 + r * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)];
     if (pair < 0) continue;
     if (HIDDEN) {
       const int col = n0 + wave_n * 32 + (lane & 31);
-      const float g = acc[0][i], u = acc[1][i];
+      const float g = acc[r][0][i], u = acc[r][1][i];
       if (col < columns) hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(g / (1.0f + expf(-g)) * u);
     } else {
       const float weight = weights[pair];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int col = n0 + j * 64 + wave_n * 32 + (lane & 31);
-        if (col < columns) out[(int64_t)pair * out_ld + col] = weight * acc[j][i];
+        if (col < columns) out[(int64_t)pair * out_ld + col] = weight * acc[r][j][i];
       }
     }
   }

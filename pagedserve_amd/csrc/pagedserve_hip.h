@@ -341,6 +341,8 @@ int ps_stream_step(float* h, const float* y, float factor, const float* bias, co
 // out[t, c] = silu(gu[t * ld + c]) * gu[t * ld + inner + c].
 int ps_silu_gate(const float* gu, int64_t ld, void* out, int64_t out_ld, int tokens, int inner,
                  int dtype, void* stream);
+// p[t * ld + first + c] = silu(...) in place for c < count.
+int ps_silu_columns(float* p, int64_t ld, int first, int count, int tokens, void* stream);
 // y += share * (rms_norm(a) * wa + rms_norm(b) * wb) over rows of width floats; a and b are cleared.
 int ps_pair_norm_mix(float* a, float* b, const float* wa, const float* wb, float eps, float share,
                      float* y, int tokens, int width, void* stream);
@@ -358,8 +360,8 @@ int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const void* w2, 
                    const float* weights, void* hidden, float* y, int tokens, int width, int inner,
                    int top, int dtype, void* stream);
 // The same for many rows in bfloat16 (width and inner multiples of 8): the (token, choice) pairs
-// are sorted by expert into tiles of 64 and multiplied on the matrix cores.  order:
-// [tiles * 64] int and tile_expert: [tiles] int scratch with tiles = ps_moe_grouped_tiles(tokens *
+// are sorted by expert into tiles of 128 and multiplied on the matrix cores.  order:
+// [tiles * 128] int and tile_expert: [tiles] int scratch with tiles = ps_moe_grouped_tiles(tokens *
 // top, experts); out: [tokens * top, width] float scratch.
 int ps_moe_grouped_tiles(int pairs, int experts);
 int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w1, const void* w2, const int* ids,

@@ -44,6 +44,16 @@ __global__ __launch_bounds__(256) void silu_gate_kernel(const float* __restrict_
   out[t * out_ld + c] = from_float<T>(g / (1.0f + expf(-g)) * u);
 }
 
+// p[t, c] <- silu(p[t, c]) for columns first .. first + count - 1 of rows ld floats apart
+__global__ __launch_bounds__(256) void silu_columns_kernel(float* __restrict__ p, int64_t ld, int first,
+                                                           int count) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= count) return;
+  float* at = p + (int64_t)blockIdx.x * ld + first + c;
+  const float v = *at;
+  *at = v / (1.0f + expf(-v));
+}
+
 // y <- y + share * (a / rms(a) * wa + b / rms(b) * wb);  a <- 0;  b <- 0.   A block per token.
 __global__ __launch_bounds__(256) void pair_norm_mix_kernel(
     float* __restrict__ a, float* __restrict__ b, const float* __restrict__ wa,
@@ -100,6 +110,15 @@ extern "C" int ps_silu_gate(const float* gu, int64_t ld, void* out, int64_t out_
   else
     hipLaunchKernelGGL(silu_gate_kernel<bf16_t>, grid, dim3(256), 0, s, gu, ld, (bf16_t*)out, out_ld, inner);
   PS_CHECK_LAUNCH("ps_silu_gate");
+  return 0;
+}
+
+extern "C" int ps_silu_columns(float* p, int64_t ld, int first, int count, int tokens, void* stream) {
+  PS_REQUIRE(tokens >= 0 && first >= 0 && count > 0 && ld >= first + count, "ps_silu_columns: bad sizes");
+  if (tokens == 0) return 0;
+  hipLaunchKernelGGL(silu_columns_kernel, dim3(tokens, (count + 255) / 256), dim3(256), 0,
+                     (hipStream_t)stream, p, ld, first, count);
+  PS_CHECK_LAUNCH("ps_silu_columns");
   return 0;
 }
 

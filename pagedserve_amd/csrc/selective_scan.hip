@@ -45,21 +45,36 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
   x[(int64_t)t * channels + c] = from_float<T>(silu_f(sum));
 }
 
-// dt[t, c] = softplus(bias[c] + sum_r low[t, r] w[c, r]).
+// dt[t, c] = softplus(bias[c] + sum_r low[t, r] w[c, r]).  A thread per channel and SS_STEP_TOKENS
+// tokens: a weight is read once for all of them.
+#define SS_STEP_TOKENS 4
 template <typename T>
 __global__ __launch_bounds__(256) void step_size_kernel(
     const float* __restrict__ low, int64_t ld, int rank, const T* __restrict__ w,
-    const float* __restrict__ bias, float* __restrict__ dt, int channels) {
-  extern __shared__ float s_low[];
-  const int t = blockIdx.x;
-  for (int r = threadIdx.x; r < rank; r += blockDim.x) s_low[r] = low[(int64_t)t * ld + r];
-  __syncthreads();
-  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
-    float z = bias ? bias[c] : 0.f;
-    const T* w_row = w + (int64_t)c * rank;
-    for (int r = 0; r < rank; ++r) z = fmaf(s_low[r], to_float<T>(w_row[r]), z);
-    dt[(int64_t)t * channels + c] = softplus_f(z);
+    const float* __restrict__ bias, float* __restrict__ dt, int tokens, int channels) {
+  extern __shared__ float s_low[];           // [SS_STEP_TOKENS][rank]
+  const int t0 = blockIdx.x * SS_STEP_TOKENS;
+  const int count = tokens - t0 < SS_STEP_TOKENS ? tokens - t0 : SS_STEP_TOKENS;
+  for (int i = threadIdx.x; i < SS_STEP_TOKENS * rank; i += blockDim.x) {
+    const int tt = i / rank;
+    s_low[i] = tt < count ? low[(int64_t)(t0 + tt) * ld + (i - tt * rank)] : 0.f;
   }
+  __syncthreads();
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= channels) return;
+  float z[SS_STEP_TOKENS];
+  const float start = bias ? bias[c] : 0.f;
+#pragma unroll
+  for (int tt = 0; tt < SS_STEP_TOKENS; ++tt) z[tt] = start;
+  const T* w_row = w + (int64_t)c * rank;
+  for (int r = 0; r < rank; ++r) {
+    const float weight = to_float<T>(w_row[r]);
+#pragma unroll
+    for (int tt = 0; tt < SS_STEP_TOKENS; ++tt) z[tt] = fmaf(s_low[tt * rank + r], weight, z[tt]);
+  }
+#pragma unroll
+  for (int tt = 0; tt < SS_STEP_TOKENS; ++tt)
+    if (tt < count) dt[(int64_t)(t0 + tt) * channels + c] = softplus_f(z[tt]);
 }
 
 // The recurrence.  A block of one wave owns 64 / LPC channels of one item and walks tokens in
@@ -306,17 +321,18 @@ extern "C" int ps_conv_silu(const float* proj, int64_t ld, int u_col, const floa
 
 extern "C" int ps_step_size(const float* low, int64_t ld, int rank, const void* w, const float* bias,
                             float* dt, int tokens, int channels, int dtype, void* stream) {
-  PS_REQUIRE(tokens >= 0 && rank > 0 && rank <= 8192 && channels > 0, "ps_step_size: bad sizes");
+  PS_REQUIRE(tokens >= 0 && rank > 0 && rank <= 2048 && channels > 0, "ps_step_size: bad sizes");
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_step_size: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const size_t lds = (size_t)rank * sizeof(float);
+  const size_t lds = (size_t)SS_STEP_TOKENS * rank * sizeof(float);
+  const dim3 grid((tokens + SS_STEP_TOKENS - 1) / SS_STEP_TOKENS, (channels + 255) / 256);
   if (dtype == PS_F32)
-    hipLaunchKernelGGL(step_size_kernel<float>, dim3(tokens), dim3(256), lds, s, low, ld, rank,
-                       (const float*)w, bias, dt, channels);
+    hipLaunchKernelGGL(step_size_kernel<float>, grid, dim3(256), lds, s, low, ld, rank,
+                       (const float*)w, bias, dt, tokens, channels);
   else
-    hipLaunchKernelGGL(step_size_kernel<bf16_t>, dim3(tokens), dim3(256), lds, s, low, ld, rank,
-                       (const bf16_t*)w, bias, dt, channels);
+    hipLaunchKernelGGL(step_size_kernel<bf16_t>, grid, dim3(256), lds, s, low, ld, rank,
+                       (const bf16_t*)w, bias, dt, tokens, channels);
   PS_CHECK_LAUNCH("ps_step_size");
   return 0;
 }

@@ -57,6 +57,7 @@ _SIGNATURES = {
                           c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "ps_stream_step": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
                        c_int, c_int, c_int, c_void_p],
+    "ps_silu_columns": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
     "ps_silu_gate": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
     "ps_pair_norm_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_int,
                          c_int, c_void_p],
@@ -1401,6 +1402,14 @@ def silu_gate(gu, out):
           inner, dtype_code(out.dtype), _stream())
 
 
+def silu_columns(rows, first, count):
+    """``rows[:, first:first + count] = silu(...)`` in place (float rows)."""
+    _check(rows, "rows", torch.float32, 2)
+    if first < 0 or count <= 0 or first + count > rows.shape[1]:
+        raise KernelError("silu_columns: the columns lie outside the rows")
+    _call("ps_silu_columns", rows.data_ptr(), _rows(rows, "rows"), first, count, rows.shape[0], _stream())
+
+
 def pair_norm_mix(a, b, weight_a, weight_b, eps, share, y, tokens, width):
     """``y += share * (rms_norm(a) * weight_a + rms_norm(b) * weight_b)``; ``a`` and ``b`` (float
     ``[tokens, width]``) are cleared."""
@@ -1433,6 +1442,7 @@ def moe_route(x, router, groups, keep, top, scale, ids, weights):
           dtype_code(x.dtype), _stream())
 
 
+MOE_TILE = 128            # pairs per tile of the sorted path (csrc/moe.hip)
 MOE_GROUPED_FROM = 128    # (token, choice) pairs from which the sorted path on the matrix cores is taken
 
 
@@ -1441,13 +1451,13 @@ def moe_grouped_supported(dtype, width, inner) -> bool:
 
 
 def moe_grouped_tiles(pairs, experts) -> int:
-    """Tiles of 64 sorted pairs that ``pairs`` pairs of ``experts`` experts can need at most."""
-    return -(-pairs // 64) + experts
+    """Tiles of ``MOE_TILE`` sorted pairs that ``pairs`` pairs of ``experts`` experts can need at most."""
+    return -(-pairs // MOE_TILE) + experts
 
 
 def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert, y):
     """``moe_experts`` for many rows in bfloat16: the pairs sorted by expert, the products on the
-    matrix cores.  ``out``: float ``[>= tokens * top, width]``, ``order``: int32 ``[>= tiles * 64]``,
+    matrix cores.  ``out``: float ``[>= tokens * top, width]``, ``order``: int32 ``[>= tiles * MOE_TILE]``,
     ``tile_expert``: int32 ``[>= tiles]`` scratch with ``tiles = moe_grouped_tiles(tokens * top, experts)``."""
     _check(x, "x", torch.bfloat16, 2)
     tokens, width = x.shape
@@ -1469,7 +1479,7 @@ def moe_experts_grouped(x, w1, w2, ids, weights, hidden, out, order, tile_expert
     _float_rows(out, "out", tokens * top, width)
     _check(order, "order", torch.int32, 1)
     _check(tile_expert, "tile_expert", torch.int32, 1)
-    if order.numel() < tiles * 64 or tile_expert.numel() < tiles:
+    if order.numel() < tiles * MOE_TILE or tile_expert.numel() < tiles:
         raise KernelError("moe_experts_grouped: the scratch for the sorted pairs is too small")
     _float_rows(y, "y", tokens, width)
     _call("ps_moe_experts_grouped", x.data_ptr(), x.stride(0), w1.data_ptr(), w2.data_ptr(), ids.data_ptr(),

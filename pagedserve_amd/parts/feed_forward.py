@@ -166,7 +166,7 @@ class MixtureOfExperts(FeedForward):
             kernels.moe_experts_grouped(
                 x, self.gate_up_weight, self.down_weight, ids, weights, hidden,
                 workspace.rows("moe_out", self.width, torch.float32, max_rows=most),
-                workspace.flat("moe_order", tiles * 64, torch.int32),
+                workspace.flat("moe_order", tiles * kernels.MOE_TILE, torch.int32),
                 workspace.flat("moe_tiles", tiles, torch.int32), residual)
         else:
             kernels.moe_experts(x, self.gate_up_weight, self.down_weight, ids, weights, hidden, residual)

@@ -161,10 +161,14 @@ class LightningAttention(Mixer):
         kernels.linear(x, self.in_weight, None, proj, packed=self.in_packed,
                        memo=site_memo(self._memo_in, workspace), shared=ctx.shared_calls)
         raw = workspace.first_rows("lightning_raw", self.v_cols, torch.float32, tokens)
+        # single tokens take the activation on their way into the recurrence; for portions, whose
+        # recurrence waits for every piece that it stages, a launch ahead of it is faster
+        if not ctx.decode_only:
+            kernels.silu_columns(proj, 0, gate_col)
         kernels.gla_scan(proj, (0, k_col, v_col), None, cache.state, raw, ctx.cu_tokens, ctx.slots,
                          self.heads, self.key_dim, self.value_dim, 1.0,
                          longest=1 if ctx.decode_only else 0, head_decay=self.head_decay,
-                         silu_inputs=True)
+                         silu_inputs=ctx.decode_only)
         gated = workspace.first_rows("lightning_out", self.v_cols, self.dtype, tokens)
         kernels.row_norm_gate(raw, self.norm_gamma, self.norm_eps,
                               proj[:, gate_col:gate_col + self.v_cols], gated)

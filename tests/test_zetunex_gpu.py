@@ -84,7 +84,7 @@ def test_gate_product_and_pair_of_norms():
 
 
 @pytest.mark.parametrize("experts,groups,keep,top", [(8, 4, 2, 3), (16, 2, 1, 3), (6, 1, 1, 6), (12, 6, 3, 1),
-                                                     (5, 5, 2, 2), (64, 8, 4, 8)])
+                                                     (5, 5, 2, 2), (64, 8, 4, 8), (128, 8, 4, 6), (66, 3, 2, 30)])
 def test_router_chooses_within_the_best_groups(experts, groups, keep, top):
     kernels = _kernels()
     g = torch.Generator().manual_seed(experts * 10 + top)
@@ -137,7 +137,7 @@ def test_experts_of_every_token(dtype, width, inner, experts, top):
 @pytest.mark.parametrize("width,inner,experts,top,tokens", [(64, 40, 5, 2, 150), (128, 96, 4, 3, 70), (72, 136, 7, 1, 333),
                                                             (256, 200, 3, 2, 64)])
 def test_experts_of_many_tokens_sorted_onto_the_matrix_cores(width, inner, experts, top, tokens):
-    """The path for many rows: pairs sorted by expert into tiles of 64 (experts with a few pairs,
+    """The path for many rows: pairs sorted by expert into tiles (experts with a few pairs,
     with more than a tile, and one with none), against the plain sum and the path for few rows."""
     kernels = _kernels()
     g = torch.Generator().manual_seed(width + inner)
@@ -158,7 +158,7 @@ def test_experts_of_many_tokens_sorted_onto_the_matrix_cores(width, inner, exper
     tiles = kernels.moe_grouped_tiles(pairs, experts)
     hidden = torch.empty((pairs, inner), dtype=dtype, device="cuda")
     out = torch.empty((pairs, width), device="cuda")
-    order = torch.empty(tiles * 64, dtype=torch.int32, device="cuda")
+    order = torch.empty(tiles * kernels.MOE_TILE, dtype=torch.int32, device="cuda")
     tile_expert = torch.empty(tiles, dtype=torch.int32, device="cuda")
     assert kernels.moe_grouped_supported(dtype, width, inner)
     kernels.moe_experts_grouped(x.cuda(), w1.cuda(), w2.cuda(), ids.cuda(), weights.cuda(), hidden, out, order,
@@ -168,9 +168,9 @@ def test_experts_of_many_tokens_sorted_onto_the_matrix_cores(width, inner, exper
     assert sorted(placed[placed >= 0].tolist()) == list(range(pairs))
     owners = tile_expert.cpu()
     flat_ids = ids.reshape(-1)
-    for place in range(0, tiles * 64, 7):
+    for place in range(0, tiles * kernels.MOE_TILE, 7):
         if int(placed[place]) >= 0:
-            assert int(owners[place // 64]) == int(flat_ids[int(placed[place])])
+            assert int(owners[place // kernels.MOE_TILE]) == int(flat_ids[int(placed[place])])
     rowwise = y0.clone().cuda()
     kernels.moe_experts(x.cuda(), w1.cuda(), w2.cuda(), ids.cuda(), weights.cuda(), torch.empty_like(hidden), rowwise)
     expected = y0.double().clone()
