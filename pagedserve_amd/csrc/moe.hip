@@ -397,8 +397,9 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
 // A tile of 128 sorted pairs times 128 weight rows of the tile's expert, k in stages of 32.
 // HIDDEN: the weight rows are 64 gate rows and the 64 up rows of the same hidden columns, and
 // hidden[pair, column] = silu(gate) * up; the rows of A are the pairs' tokens (pair / top).
-// Otherwise: 128 output columns, out[pair, column] = weights[pair] * sum; the rows of A are the
-// pairs' hidden rows.  Four waves, 2 x 2: a wave has 64 pairs and two times 32 weight rows.
+// Otherwise: 64 output columns (so that the narrower product still gives every compute unit a
+// block), out[pair, column] = weights[pair] * sum; the rows of A are the pairs' hidden rows.
+// Four waves, 2 x 2: a wave has 64 pairs and 32 weight rows, twice in the first case.
 template <bool HIDDEN>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t expert_stride,
@@ -413,7 +414,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave >> 1, wave_n = wave & 1;
   const int columns = HIDDEN ? w_rows / 2 : w_rows;      // output columns
-  const int n0 = blockIdx.y * (HIDDEN ? 64 : 128);
+  constexpr int NJ = HIDDEN ? 2 : 1;                     // runs of 64 weight rows in a stage
+  const int n0 = blockIdx.y * 64;
   if (tid < MOE_TILE) s_pair[tid] = order[blockIdx.x * MOE_TILE + tid];
   __syncthreads();
   // staging: 16-byte chunks, 4 per row; A and W: 128 rows each, two chunks a thread
@@ -432,7 +434,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     int row;
     if (HIDDEN) row = (local < 64 ? 0 : columns) + n0 + (local & 63);
     else row = n0 + local;
-    w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : row < w_rows;
+    w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : (local < 64 && row < w_rows);
     w_src[i] = w + (int64_t)e * expert_stride + (int64_t)(w_ok[i] ? row : 0) * k + chunk;
   }
   uint4 stage_a[2], stage_w[2];
@@ -444,8 +446,10 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     for (int i = 0; i < 2; ++i) {
       stage_a[i] = *reinterpret_cast<const uint4*>(a_src[i] + kk);
       if (!(k_ok && a_ok[i])) stage_a[i] = zero;
-      stage_w[i] = *reinterpret_cast<const uint4*>(w_src[i] + kk);
-      if (!(k_ok && w_ok[i])) stage_w[i] = zero;
+      if (i < NJ) {
+        stage_w[i] = *reinterpret_cast<const uint4*>(w_src[i] + kk);
+        if (!(k_ok && w_ok[i])) stage_w[i] = zero;
+      }
     }
   };
   auto store_lds = [&](int buffer) {
@@ -453,7 +457,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       *reinterpret_cast<uint4*>(&lds[buffer][i * 64 * MOE_LDS_STRIDE + offset]) = stage_a[i];
-      *reinterpret_cast<uint4*>(&lds[buffer][(MOE_TILE + i * 64) * MOE_LDS_STRIDE + offset]) = stage_w[i];
+      if (i < NJ)
+        *reinterpret_cast<uint4*>(&lds[buffer][(MOE_TILE + i * 64) * MOE_LDS_STRIDE + offset]) = stage_w[i];
     }
   };
   moe_f32x16 acc[2][2];      // [rows of 32 pairs][weight rows]
@@ -479,13 +484,13 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
         fa[r] = *reinterpret_cast<const uint4*>(
             &stage[(wave_m * 64 + r * 32 + (lane & 31)) * MOE_LDS_STRIDE + kbyte]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < NJ; ++j)
         fw[j] = *reinterpret_cast<const uint4*>(
             &stage[(MOE_TILE + j * 64 + wave_n * 32 + (lane & 31)) * MOE_LDS_STRIDE + kbyte]);
 #pragma unroll
       for (int r = 0; r < 2; ++r)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
           acc[r][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
               *reinterpret_cast<const moe_bf16x8*>(&fa[r]), *reinterpret_cast<const moe_bf16x8*>(&fw[j]),
               acc[r][j], 0, 0, 0);
@@ -504,12 +509,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       const float g = acc[r][0][i], u = acc[r][1][i];
       if (col < columns) hidden[(int64_t)pair * columns + col] = from_float<bf16_t>(g / (1.0f + expf(-g)) * u);
     } else {
-      const float weight = weights[pair];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int col = n0 + j * 64 + wave_n * 32 + (lane & 31);
-        if (col < columns) out[(int64_t)pair * out_ld + col] = weight * acc[r][j][i];
-      }
+      const int col = n0 + wave_n * 32 + (lane & 31);
+      if (col < columns) out[(int64_t)pair * out_ld + col] = weights[pair] * acc[r][0][i];
     }
   }
 }
@@ -584,7 +585,7 @@ extern "C" int ps_moe_experts_grouped(const void* x, int64_t x_ld, const void* w
                      (const bf16_t*)x, x_ld, (const bf16_t*)w1, (int64_t)2 * inner * width, 2 * inner,
                      width, order, tile_expert, top, weights, (bf16_t*)hidden, (float*)nullptr,
                      (int64_t)0);
-  hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3(tiles, (width + 127) / 128), dim3(256), 0, s,
+  hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3(tiles, (width + 63) / 64), dim3(256), 0, s,
                      (const bf16_t*)hidden, (int64_t)inner, (const bf16_t*)w2, (int64_t)width * inner,
                      width, inner, order, tile_expert, top, weights, (bf16_t*)nullptr, out,
                      (int64_t)width);
