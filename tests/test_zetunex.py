@@ -91,8 +91,9 @@ def test_every_parameter_has_a_source_and_every_tensor_a_parameter(tmp_path):
             if layer["mlp"] is not None and layer["mlp"]["kind"] == "moe":
                 part = model.blocks[index].feed_forward
                 ff = layer["mlp"]["expert"]["ff"]
+                last = layer["mlp"]["router"]["experts"] - 1
                 assert torch.equal(part.gate_up_weight[1, ff:], tensors[f"l{index}.mlp.e1.up"])
-                assert torch.equal(part.down_weight[2], tensors[f"l{index}.mlp.e2.down"])
+                assert torch.equal(part.down_weight[last], tensors[f"l{index}.mlp.e{last}.down"])
         if raw.get("loop"):
             assert torch.equal(model.pass_table, tensors["loop.step"])
 

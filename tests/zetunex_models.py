@@ -64,8 +64,19 @@ MODEL_D = {
     "layers": [_parallel(3, 1, 40, 8, 0.1, 500, 24, 130, 2, 1, _moe(12, 3, 6, 3, 0.8, 20)),
                _lightning(1, 40, 72, [0.93], _moe(6, 4, 3, 2, 1.0, 24))],
 }
+# the smallest of everything: a window of one token (a query sees itself only), one state per
+# channel, a single head, every expert of the one group chosen, a pass that is made once, sizes
+# that are multiples of nothing, a recurrent layer without a feed-forward first
+MODEL_E = {
+    "architecture": "Zetunex", "vocab": 33, "width": 24, "norm": {"eps": 1e-4}, "residual_mult": 0.25,
+    "loop": {"start": 1, "stop": 2, "times": 1},
+    "layers": [_lightning(1, 8, 4, [0.75], None),
+               _parallel(1, 1, 12, 20, 0.5, 1, 10, 1, 5, 5, _moe(2, 2, 1, 1, 3.0, 7)),
+               _parallel(6, 3, 4, 4, 0.7, 2, 18, 3, 2, 3, _dense(9))],
+}
 # name -> (configuration, page size, seed)
-MODELS = {"A": (MODEL_A, 8, 0), "B": (MODEL_B, 16, 1), "C": (MODEL_C, 16, 2), "D": (MODEL_D, 4, 3)}
+MODELS = {"A": (MODEL_A, 8, 0), "B": (MODEL_B, 16, 1), "C": (MODEL_C, 16, 2), "D": (MODEL_D, 4, 3),
+          "E": (MODEL_E, 2, 4)}
 
 
 def write_folder(folder, raw, tensors):
