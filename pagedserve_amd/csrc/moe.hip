@@ -393,6 +393,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float moe_f32x16;
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
 #define MOE_LDS_STRIDE 80   // bytes between rows of a stage (64 bytes of k, padded)
+#define MOE_DEPTH 4         // k tiles whose global loads are in flight
 
 // A tile of 128 sorted pairs times 128 weight rows of the tile's expert, k in stages of 32.
 // HIDDEN: the weight rows are 64 gate rows and the 64 up rows of the same hidden columns, and
@@ -437,9 +438,10 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     w_ok[i] = HIDDEN ? n0 + (local & 63) < columns : (local < 64 && row < w_rows);
     w_src[i] = w + (int64_t)e * expert_stride + (int64_t)(w_ok[i] ? row : 0) * k + chunk;
   }
-  uint4 stage_a[2], stage_w[2];
+  // a ring of MOE_DEPTH stages in registers keeps that many k tiles' loads in flight
+  uint4 ring_a[MOE_DEPTH][2], ring_w[MOE_DEPTH][2];
   const uint4 zero = {0u, 0u, 0u, 0u};
-  auto load_global = [&](int k0) {
+  auto load_global = [&](uint4* stage_a, uint4* stage_w, int k0) {
     const bool k_ok = k0 + chunk < k;
     const int kk = k_ok ? k0 : 0;
 #pragma unroll
@@ -452,7 +454,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       }
     }
   };
-  auto store_lds = [&](int buffer) {
+  auto store_lds = [&](int buffer, const uint4* stage_a, const uint4* stage_w) {
     const int offset = a_row * MOE_LDS_STRIDE + (tid & 3) * 16;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -469,12 +471,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[r][j][i] = 0.f;
   const int k_tiles = (k + 31) / 32;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    if (kt + 1 < k_tiles) load_global((kt + 1) * 32);
-    const unsigned char* stage = lds[kt & 1];
+  auto compute = [&](int buffer) {
+    const unsigned char* stage = lds[buffer];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int kbyte = half * 32 + (lane >> 5) * 16;
@@ -495,8 +493,24 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
               *reinterpret_cast<const moe_bf16x8*>(&fa[r]), *reinterpret_cast<const moe_bf16x8*>(&fw[j]),
               acc[r][j], 0, 0, 0);
     }
-    if (kt + 1 < k_tiles) store_lds((kt + 1) & 1);
-    __syncthreads();
+  };
+#pragma unroll
+  for (int d = 0; d < MOE_DEPTH; ++d) load_global(ring_a[d], ring_w[d], d * 32);
+  store_lds(0, ring_a[0], ring_w[0]);
+  __syncthreads();
+  for (int kt0 = 0; kt0 < k_tiles; kt0 += MOE_DEPTH) {
+#pragma unroll
+    for (int d = 0; d < MOE_DEPTH; ++d) {
+      const int kt = kt0 + d;
+      if (kt < k_tiles) {
+        // stage d held tile kt, which is in LDS already: refill it with tile kt + MOE_DEPTH
+        load_global(ring_a[d], ring_w[d], (kt + MOE_DEPTH) * 32);
+        compute(kt & 1);
+        // tile kt + 1 left MOE_DEPTH - 1 iterations ago
+        store_lds((kt + 1) & 1, ring_a[(d + 1) % MOE_DEPTH], ring_w[(d + 1) % MOE_DEPTH]);
+        __syncthreads();
+      }
+    }
   }
   // element i of an accumulator: row (i / 4) * 8 + (lane / 32) * 4 + i % 4, column lane % 32
 #pragma unroll
@@ -536,12 +550,14 @@ extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_moe_experts: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  constexpr int ROWS = 4;
-  const dim3 grid1(tokens, (inner + 4 * ROWS - 1) / (4 * ROWS), top);
-  const dim3 grid2(tokens, (width + 4 * ROWS - 1) / (4 * ROWS));
   const bool wide1 = width % 8 == 0 && x_ld % 8 == 0, wide2 = inner % 8 == 0;
-#define PS_MOE_ROWS(T)                                                                             \
+  // hidden columns / output columns per wave: four, or two while that still leaves the chip
+  // short of blocks (a handful of decoded tokens)
+  const bool few = (int64_t)tokens * ((width + 15) / 16) < 4 * ps_compute_units();
+#define PS_MOE_ROWS(T, ROWS)                                                                       \
   do {                                                                                             \
+    const dim3 grid1(tokens, (inner + 4 * ROWS - 1) / (4 * ROWS), top);                            \
+    const dim3 grid2(tokens, (width + 4 * ROWS - 1) / (4 * ROWS));                                 \
     if (wide1)                                                                                     \
       hipLaunchKernelGGL((moe_hidden_wide_kernel<T, ROWS>), grid1, dim3(256), (size_t)width * 4, s, \
                          (const T*)x, x_ld, (const T*)w1, ids, (T*)hidden, width, inner);          \
@@ -555,8 +571,13 @@ extern "C" int ps_moe_experts(const void* x, int64_t x_ld, const void* w1, const
       hipLaunchKernelGGL((moe_down_kernel<T, ROWS>), grid2, dim3(256), (size_t)top * inner * 4, s, \
                          (const T*)hidden, (const T*)w2, ids, weights, y, width, inner, top);      \
   } while (0)
-  if (dtype == PS_F32) PS_MOE_ROWS(float);
-  else PS_MOE_ROWS(bf16_t);
+  if (dtype == PS_F32) {
+    if (few) PS_MOE_ROWS(float, 2);
+    else PS_MOE_ROWS(float, 4);
+  } else {
+    if (few) PS_MOE_ROWS(bf16_t, 2);
+    else PS_MOE_ROWS(bf16_t, 4);
+  }
 #undef PS_MOE_ROWS
   PS_CHECK_LAUNCH("ps_moe_experts");
   return 0;

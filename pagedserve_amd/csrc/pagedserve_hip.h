@@ -325,12 +325,15 @@ int ps_step_size(const float* low, int64_t ld, int rank, const void* w, const fl
 // records / sums (or null for both): scratch of (pieces + items) * channels * states and
 // (pieces + items) * channels floats with pieces = ps_selective_pieces(tokens, items); with them
 // the items are cut into pieces that run side by side (for steps with long portions).
+// dt null: the step sizes are worked out on the way, softplus(step_bias[c] + sum_r bc[t * bc_ld +
+// low_col + r] step_w[c, r]) with step_w [channels, rank] of the storage type, rank <= 256.
 int ps_selective_pieces(int tokens, int items);
 int ps_selective_scan(const void* x, const float* dt, const float* bc, int64_t bc_ld, int b_col,
                       int c_col, const float* proj, int64_t ld, int u_col, int z_col,
                       const float* a_log, const float* skip, float* state, void* y,
                       const int* cu_tokens, const int* slots, int items, int channels, int states,
-                      int taps, int tokens, float* records, float* sums, int dtype, void* stream);
+                      int taps, int tokens, float* records, float* sums, const void* step_w,
+                      const float* step_bias, int low_col, int rank, int dtype, void* stream);
 
 // ---- a stream whose sublayers add into a scratch row ------------------------------------------
 // h += factor * y + bias (y, bias: null for none); zero[...] = 0 (may be y); if gamma:

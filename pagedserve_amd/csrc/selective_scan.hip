@@ -95,6 +95,11 @@ struct ScanArgs {
   const int* cu_tokens;
   const int* slots;
   int channels, states, taps;
+  // where dt is null, the step sizes are worked out on the way: softplus(step_bias[c] + sum_r
+  // bc[t, low_col + r] step_w[c, r]) with weights of the storage type
+  const void* step_w;
+  const float* step_bias;
+  int low_col, rank;
 };
 
 // Tokens first .. last - 1 of one item for the block's channels, from the states in S.  EMIT:
@@ -107,6 +112,10 @@ __device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T
   const int part = lane % LPC;
   const int states = p.states, channels = p.channels;
   const float d_skip = EMIT ? p.skip[cc] : 0.f;
+  const bool own_steps = p.dt == nullptr;
+  const T* step_row = (const T*)p.step_w + (int64_t)cc * p.rank;
+  const float step_bias = own_steps && p.step_bias != nullptr ? p.step_bias[cc] : 0.f;
+  float* s_low = s_bc + SS_CHUNK * 2 * states;       // [SS_CHUNK][rank], only with own step sizes
   float steps = 0.f;
   for (int base = first; base < last; base += SS_CHUNK) {
     const int count = (last - base) < SS_CHUNK ? (last - base) : SS_CHUNK;
@@ -116,10 +125,24 @@ __device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T
       const int n = idx - tt * 2 * states;
       s_bc[idx] = p.bc[(int64_t)(base + tt) * p.bc_ld + (n < states ? p.b_col + n : p.c_col + n - states)];
     }
+    if (own_steps) {
+      for (int idx = lane; idx < count * p.rank; idx += 64) {
+        const int tt = idx / p.rank;
+        s_low[idx] = p.bc[(int64_t)(base + tt) * p.bc_ld + p.low_col + (idx - tt * p.rank)];
+      }
+    }
     __syncthreads();
     for (int tt = 0; tt < count; ++tt) {
       const int64_t t = base + tt;
-      const float step = p.dt[t * channels + cc];
+      float step;
+      if (own_steps) {
+        // the channel's lanes share the low-rank sum
+        float z = 0.f;
+        for (int r = part; r < p.rank; r += LPC) z = fmaf(s_low[tt * p.rank + r], to_float<T>(step_row[r]), z);
+        step = softplus_f(lanes_sum<LPC>(z) + step_bias);
+      } else {
+        step = p.dt[t * channels + cc];
+      }
       const float xv = to_float<T>(x[t * channels + cc]);
       const float* b_row = s_bc + tt * 2 * states;
       const float* c_row = b_row + states;
@@ -349,16 +372,19 @@ extern "C" int ps_selective_scan(const void* x, const float* dt, const float* bc
                                  int z_col, const float* a_log, const float* skip, float* state,
                                  void* y, const int* cu_tokens, const int* slots, int items,
                                  int channels, int states, int taps, int tokens, float* records,
-                                 float* sums, int dtype, void* stream) {
+                                 float* sums, const void* step_w, const float* step_bias,
+                                 int low_col, int rank, int dtype, void* stream) {
   PS_REQUIRE(items >= 0 && channels > 0 && states > 0 && taps >= 1, "ps_selective_scan: bad sizes");
   PS_REQUIRE(states <= 256, "ps_selective_scan: %d states per channel, at most 256", states);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_selective_scan: unknown dtype %d", dtype);
   PS_REQUIRE((records == nullptr) == (sums == nullptr), "ps_selective_scan: records and sums go together");
+  PS_REQUIRE(dt != nullptr || (step_w != nullptr && rank > 0 && rank <= 256 && low_col >= 0),
+             "ps_selective_scan: neither step sizes nor weights (of rank 1..256) to work them out");
   if (items == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const size_t lds = (size_t)SS_CHUNK * 2 * states * sizeof(float);
+  const size_t lds = (size_t)SS_CHUNK * (2 * states + (dt == nullptr ? rank : 0)) * sizeof(float);
   const ScanArgs p = {dt, bc, bc_ld, b_col, c_col, proj, ld, u_col, z_col, a_log, skip, state,
-                      cu_tokens, slots, channels, states, taps};
+                      cu_tokens, slots, channels, states, taps, step_w, step_bias, low_col, rank};
   const int pieces = ps_selective_pieces(tokens, items);
 #define PS_LAUNCH_SS_T(T, LPC, SPL)                                                               \
   do {                                                                                            \

@@ -54,7 +54,8 @@ _SIGNATURES = {
                      c_void_p],
     "ps_selective_scan": [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                           c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
+                          c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_int, c_void_p],
     "ps_stream_step": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
                        c_int, c_int, c_int, c_void_p],
     "ps_silu_columns": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
@@ -1318,6 +1319,7 @@ def step_size(low, w, bias, dt):
 
 
 SCAN_PIECE = 32     # tokens of a piece of the selective scan's launch in pieces
+SCAN_FUSED_RANK = 256   # largest rank of the step-size projection that the scan works out itself
 
 
 def selective_scan_records(tokens, items, channels, states):
@@ -1328,18 +1330,33 @@ def selective_scan_records(tokens, items, channels, states):
 
 
 def selective_scan(x, dt, bc, b_col, c_col, proj, u_col, z_col, a_log, skip, state, y, cu_tokens,
-                   slots, taps, scratch=None):
+                   slots, taps, scratch=None, step_weights=None):
     """The selective recurrence over the step's items (``csrc/pagedserve_hip.h: ps_selective_scan``);
     ``state``: float ``[slots, channels, states + taps - 1]``.  ``scratch = (records, sums)``: float
     buffers of at least ``selective_scan_records(...)`` elements; with them the items are cut into
-    pieces that run side by side (three launches: for steps with long portions)."""
+    pieces that run side by side (three launches: for steps with long portions).
+    ``dt=None`` with ``step_weights = (low_col, w, bias)``: the step sizes are worked out inside the
+    launch from the columns ``low_col...`` of ``bc`` (``w``: ``[channels, rank]`` of x's dtype, rank <= 256)."""
     _check(x, "x", ndim=2)
     tokens, channels = x.shape
     _check(a_log, "a_log", torch.float32, 2)
     states = a_log.shape[1]
     if a_log.shape[0] != channels or not a_log.is_contiguous() or not x.is_contiguous():
         raise KernelError("selective_scan: a_log must be contiguous [channels, states]")
-    _float_rows(dt, "dt", tokens, channels)
+    low_col, step_w, step_bias, rank = 0, None, None, 0
+    if dt is not None:
+        _float_rows(dt, "dt", tokens, channels)
+    else:
+        if step_weights is None:
+            raise KernelError("selective_scan: neither step sizes nor the weights to work them out")
+        low_col, step_w, step_bias = step_weights
+        _check(step_w, "step weights", x.dtype, 2)
+        rank = step_w.shape[1]
+        if (step_w.shape[0] != channels or not step_w.is_contiguous() or rank > SCAN_FUSED_RANK
+                or low_col < 0 or low_col + rank > bc.shape[1]):
+            raise KernelError("selective_scan: step weights must be contiguous [channels, rank <= 256]")
+        if step_bias is not None:
+            _float_vector(step_bias, "step bias", channels)
     _float_vector(skip, "skip", channels)
     _check(bc, "bc", torch.float32, 2)
     _check(proj, "proj", torch.float32, 2)
@@ -1360,10 +1377,11 @@ def selective_scan(x, dt, bc, b_col, c_col, proj, u_col, z_col, a_log, skip, sta
         _check(sums, "sums", torch.float32, 1)
         if records.numel() < need[0] or sums.numel() < need[1]:
             raise KernelError("selective_scan: the scratch for the pieces is too small")
-    _call("ps_selective_scan", x.data_ptr(), dt.data_ptr(), bc.data_ptr(), bc.stride(0), b_col, c_col,
+    _call("ps_selective_scan", x.data_ptr(), _ptr(dt), bc.data_ptr(), bc.stride(0), b_col, c_col,
           proj.data_ptr(), proj.stride(0), u_col, z_col, a_log.data_ptr(), skip.data_ptr(),
           state.data_ptr(), y.data_ptr(), cu_tokens.data_ptr(), slots.data_ptr(), items, channels,
-          states, taps, tokens, _ptr(records), _ptr(sums), dtype_code(x.dtype), _stream())
+          states, taps, tokens, _ptr(records), _ptr(sums), _ptr(step_w), _ptr(step_bias), low_col, rank,
+          dtype_code(x.dtype), _stream())
 
 
 def stream_step(h, tokens, width, add=None, bias=None, norm=None, zero=None):

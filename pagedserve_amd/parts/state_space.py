@@ -82,12 +82,18 @@ class SelectiveScan(Mixer):
         low = workspace.first_rows("scan_low", rank + 2 * states, torch.float32, tokens)
         kernels.linear(activated, self.x_weight, None, low, packed=self.x_packed,
                        memo=site_memo(self._memo_x, workspace), shared=ctx.shared_calls)
-        dt = workspace.first_rows("scan_dt", inner, torch.float32, tokens)
-        kernels.step_size(low[:, :rank], self.dt_weight, self.dt_bias, dt)
         y = workspace.first_rows("scan_y", inner, self.dtype, tokens)
         scratch = None
         items = ctx.slots.numel()
-        if tokens - items >= self.PIECES_FROM:
+        pieces = tokens - items >= self.PIECES_FROM
+        dt = step_weights = None
+        if pieces or rank > kernels.SCAN_FUSED_RANK:
+            dt = workspace.first_rows("scan_dt", inner, torch.float32, tokens)
+            kernels.step_size(low[:, :rank], self.dt_weight, self.dt_bias, dt)
+        else:
+            # decoded tokens and short portions: the recurrence works its step sizes out itself
+            step_weights = (0, self.dt_weight, self.dt_bias)
+        if pieces:
             # some item brings a long portion: pieces of it run side by side.  The scratch is
             # asked for at its largest, so that it never moves under recorded launches.
             most = kernels.selective_scan_records(workspace.max_rows, cache.state.shape[0], inner, states)
@@ -95,7 +101,7 @@ class SelectiveScan(Mixer):
                        workspace.flat("scan_sums", most[1], torch.float32))
         kernels.selective_scan(activated, dt, low, rank, rank + states, proj, 0, inner, self.a_log,
                                self.skip, cache.state, y, ctx.cu_tokens, ctx.slots, self.taps,
-                               scratch=scratch)
+                               scratch=scratch, step_weights=step_weights)
         kernels.linear(y, self.out_weight, None, residual, epilogue="residual",
                        packed=self.out_packed, memo=site_memo(self._memo_out, workspace),
                        shared=ctx.shared_calls)

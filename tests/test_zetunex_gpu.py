@@ -217,7 +217,7 @@ def test_selective_scan_in_one_go_in_pieces_and_in_reused_slots(dtype, channels,
         cu.append(cu[-1] + length)
     tok_item = _ints([n for n, length in enumerate(lengths) for _ in range(length)])
 
-    def run(rows, state, cu_list, slot_list, items, pieces=False):
+    def run(rows, state, cu_list, slot_list, items, pieces=False, own_steps=False):
         count = rows.stop - rows.start
         dproj, dlow = proj[rows].cuda(), low[rows].cuda()
         x = torch.empty((count, channels), dtype=dtype, device="cuda")
@@ -230,8 +230,11 @@ def test_selective_scan_in_one_go_in_pieces_and_in_reused_slots(dtype, channels,
         if pieces:
             sizes = kernels.selective_scan_records(count, len(slot_list), channels, states)
             scratch = tuple(torch.full((size,), float("nan"), device="cuda") for size in sizes)
-        kernels.selective_scan(x, dt, dlow, b_col, c_col, dproj, u_col, z_col, a_log.cuda(), skip.cuda(),
-                               state, y, _ints(cu_list), _ints(slot_list), taps, scratch=scratch)
+        # (own_steps: the launch works the step sizes out itself instead of reading them)
+        kernels.selective_scan(x, None if own_steps else dt, dlow, b_col, c_col, dproj, u_col, z_col,
+                               a_log.cuda(), skip.cuda(), state, y, _ints(cu_list), _ints(slot_list), taps,
+                               scratch=scratch,
+                               step_weights=(1, dt_w.cuda(), dt_b.cuda()) if own_steps else None)
         return x, dt, y
 
     x, dt, y = run(slice(0, total), state, cu, slots, tok_item)
@@ -273,7 +276,8 @@ def test_selective_scan_in_one_go_in_pieces_and_in_reused_slots(dtype, channels,
     state[0].zero_()
     cursor, pieces = 0, []
     for size in (1, 2, 1, 7, 16, 17, 1):
-        _, _, piece = run(slice(cursor, cursor + size), state, [0, size], [0], _ints([0] * size))
+        _, _, piece = run(slice(cursor, cursor + size), state, [0, size], [0], _ints([0] * size),
+                          own_steps=size != 7)
         pieces.append(piece)
         cursor += size
     assert cursor == lengths[0]
