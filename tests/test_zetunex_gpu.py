@@ -110,7 +110,7 @@ def test_router_chooses_within_the_best_groups(experts, groups, keep, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width,inner,experts,top", [(48, 20, 5, 2), (128, 96, 4, 3), (72, 130, 3, 1)])
+@pytest.mark.parametrize("width,inner,experts,top", [(48, 20, 5, 2), (128, 96, 4, 3), (72, 130, 3, 1), (44, 24, 5, 2)])
 def test_experts_of_every_token(dtype, width, inner, experts, top):
     kernels = _kernels()
     g = torch.Generator().manual_seed(width + inner)
