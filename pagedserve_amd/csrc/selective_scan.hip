@@ -104,18 +104,30 @@ struct ScanArgs {
 
 // Tokens first .. last - 1 of one item for the block's channels, from the states in S.  EMIT:
 // the outputs are written; else only the states move, and the lanes get the sum of the step sizes.
+// Everything that a token's step reads waits in LDS, SS_CHUNK tokens at a time (B and C, the
+// block's channels of the step sizes, inputs and gates, loaded by all lanes side by side), so
+// that the walk from token to token never waits for memory; the outputs of a chunk leave
+// together, gated, after its walk.
+// LDS: [SS_CHUNK][2 * states] | [SS_CHUNK][rank] (own step sizes only) | 4 x [SS_CHUNK][CPB].
 template <typename T, int LPC, int SPL, bool EMIT>
 __device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T* __restrict__ y,
                                    int first, int last, int c, int cc, bool live, float (&S)[SPL],
                                    const float (&A)[SPL], float* s_bc) {
+  constexpr int CPB = 64 / LPC;
   const int lane = threadIdx.x;
   const int part = lane % LPC;
+  const int mine = lane / LPC;                       // the lane's channel within the block
   const int states = p.states, channels = p.channels;
   const float d_skip = EMIT ? p.skip[cc] : 0.f;
   const bool own_steps = p.dt == nullptr;
   const T* step_row = (const T*)p.step_w + (int64_t)cc * p.rank;
   const float step_bias = own_steps && p.step_bias != nullptr ? p.step_bias[cc] : 0.f;
   float* s_low = s_bc + SS_CHUNK * 2 * states;       // [SS_CHUNK][rank], only with own step sizes
+  float* s_dt = s_low + (own_steps ? SS_CHUNK * p.rank : 0);
+  float* s_x = s_dt + SS_CHUNK * CPB;
+  float* s_z = s_x + SS_CHUNK * CPB;
+  float* s_y = s_z + SS_CHUNK * CPB;
+  const int c0 = c - mine;                           // the block's first channel
   float steps = 0.f;
   for (int base = first; base < last; base += SS_CHUNK) {
     const int count = (last - base) < SS_CHUNK ? (last - base) : SS_CHUNK;
@@ -131,9 +143,16 @@ __device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T
         s_low[idx] = p.bc[(int64_t)(base + tt) * p.bc_ld + p.low_col + (idx - tt * p.rank)];
       }
     }
+    for (int idx = lane; idx < count * CPB; idx += 64) {
+      const int tt = idx / CPB;
+      const int64_t t = base + tt;
+      const int channel = c0 + (idx - tt * CPB) < channels ? c0 + (idx - tt * CPB) : channels - 1;
+      if (!own_steps) s_dt[idx] = p.dt[t * channels + channel];
+      s_x[idx] = to_float<T>(x[t * channels + channel]);
+      if (EMIT) s_z[idx] = p.proj[t * p.ld + p.z_col + channel];
+    }
     __syncthreads();
     for (int tt = 0; tt < count; ++tt) {
-      const int64_t t = base + tt;
       float step;
       if (own_steps) {
         // the channel's lanes share the low-rank sum
@@ -141,9 +160,9 @@ __device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T
         for (int r = part; r < p.rank; r += LPC) z = fmaf(s_low[tt * p.rank + r], to_float<T>(step_row[r]), z);
         step = softplus_f(lanes_sum<LPC>(z) + step_bias);
       } else {
-        step = p.dt[t * channels + cc];
+        step = s_dt[tt * CPB + mine];
       }
-      const float xv = to_float<T>(x[t * channels + cc]);
+      const float xv = s_x[tt * CPB + mine];
       const float* b_row = s_bc + tt * 2 * states;
       const float* c_row = b_row + states;
       const float sx = step * xv;
@@ -159,13 +178,20 @@ __device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T
       }
       if (EMIT) {
         sum = lanes_sum<LPC>(sum);
-        if (part == 0 && live) {
-          const float z = p.proj[t * p.ld + p.z_col + c];
-          y[t * channels + c] = from_float<T>(fmaf(d_skip, xv, sum) * silu_f(z));
-        }
+        if (part == 0) s_y[tt * CPB + mine] = fmaf(d_skip, xv, sum);
+      }
+    }
+    if (EMIT) {
+      __syncthreads();
+      for (int idx = lane; idx < count * CPB; idx += 64) {
+        const int tt = idx / CPB;
+        const int channel = c0 + (idx - tt * CPB);
+        if (channel < channels)
+          y[(int64_t)(base + tt) * channels + channel] = from_float<T>(s_y[idx] * silu_f(s_z[idx]));
       }
     }
   }
+  (void)live;
   return steps;
 }
 
@@ -382,13 +408,14 @@ extern "C" int ps_selective_scan(const void* x, const float* dt, const float* bc
              "ps_selective_scan: neither step sizes nor weights (of rank 1..256) to work them out");
   if (items == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const size_t lds = (size_t)SS_CHUNK * (2 * states + (dt == nullptr ? rank : 0)) * sizeof(float);
+  const int staged = 2 * states + (dt == nullptr ? rank : 0);     // floats per token beside the channels' own
   const ScanArgs p = {dt, bc, bc_ld, b_col, c_col, proj, ld, u_col, z_col, a_log, skip, state,
                       cu_tokens, slots, channels, states, taps, step_w, step_bias, low_col, rank};
   const int pieces = ps_selective_pieces(tokens, items);
 #define PS_LAUNCH_SS_T(T, LPC, SPL)                                                               \
   do {                                                                                            \
     const int blocks = (channels + 64 / LPC - 1) / (64 / LPC);                                    \
+    const size_t lds = (size_t)SS_CHUNK * (staged + 4 * (64 / LPC)) * sizeof(float);               \
     if (records == nullptr) {                                                                     \
       hipLaunchKernelGGL((selective_scan_kernel<T, LPC, SPL>), dim3(items, blocks), dim3(64), lds, s, \
                          p, (const T*)x, (T*)y);                                                  \
