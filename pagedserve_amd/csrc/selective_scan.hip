@@ -20,6 +20,23 @@ __device__ inline float silu_f(float v) { return v / (1.0f + expf(-v)); }
 // softplus(v) = max(v, 0) + log1p(exp(-|v|))
 __device__ inline float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
+// exp(rate * step) of the recurrence's decays, rate = A (or A * log2(e), see decay_rate).  The
+// float engine takes the library's exponential; the bfloat16 engine, whose inputs carry three
+// decimal digits, takes the hardware's base-2 exponential (one instruction after the product
+// instead of a dozen: the walk over the tokens is bound by the instructions it issues).
+template <typename T>
+__device__ inline float decay_rate(float a);
+template <>
+__device__ inline float decay_rate<float>(float a) { return a; }
+template <>
+__device__ inline float decay_rate<bf16_t>(float a) { return a * 1.4426950408889634f; }
+template <typename T>
+__device__ inline float decay_of(float rate, float step);
+template <>
+__device__ inline float decay_of<float>(float rate, float step) { return expf(rate * step); }
+template <>
+__device__ inline float decay_of<bf16_t>(float rate, float step) { return __builtin_amdgcn_exp2f(rate * step); }
+
 // x[t, c] = silu(conv(u)[t, c]): a thread per (token, channel).  Inputs before the step's first
 // token of the item come from the slot (zeros for a new request: the slot was cleared).
 template <typename T>
@@ -172,7 +189,7 @@ __device__ inline float scan_range(const ScanArgs& p, const T* __restrict__ x, T
       for (int i = 0; i < SPL; ++i) {
         const int n = part + i * LPC;
         if (n < states) {
-          S[i] = fmaf(expf(step * A[i]), S[i], sx * b_row[n]);
+          S[i] = fmaf(decay_of<T>(A[i], step), S[i], sx * b_row[n]);
           if (EMIT) sum = fmaf(S[i], c_row[n], sum);
         }
       }
@@ -225,7 +242,7 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(ScanArgs p, const T*
   for (int i = 0; i < SPL; ++i) {
     const int n = part + i * LPC;
     S[i] = n < p.states ? mine[n] : 0.f;
-    A[i] = n < p.states ? -expf(p.a_log[(int64_t)cc * p.states + n]) : 0.f;
+    A[i] = n < p.states ? decay_rate<T>(-expf(p.a_log[(int64_t)cc * p.states + n])) : 0.f;
   }
   scan_range<T, LPC, SPL, true>(p, x, y, t0, t1, c, cc, live, S, A, s_bc);
   if (!live) return;
@@ -296,7 +313,7 @@ __global__ __launch_bounds__(64) void selective_pieces_kernel(ScanArgs p, const 
 #pragma unroll
   for (int i = 0; i < SPL; ++i) {
     const int n = part + i * LPC;
-    A[i] = n < p.states ? -expf(p.a_log[(int64_t)cc * p.states + n]) : 0.f;
+    A[i] = n < p.states ? decay_rate<T>(-expf(p.a_log[(int64_t)cc * p.states + n])) : 0.f;
     S[i] = (EMIT && n < p.states) ? record[n] : 0.f;
   }
   if (!EMIT && at.piece == 0 && live) {
