@@ -228,6 +228,72 @@ extern "C" int ps_row_norm_gate(const float* o, const float* w, float eps, const
   return 0;
 }
 
+// ---- long portions in pieces that run side by side (recurrences with one decay per head) ----
+// The recurrence is linear in the state: a piece of n tokens takes S to d^n S + E, with E what
+// it leaves from a zero state.  So the items of a step are cut into pieces, every piece runs
+// the recurrence kernel as an item of its own with a state of its own (first from zero, which
+// leaves E there; then, once ps_decay_join has put every piece's true start in E's place, again,
+// now for the outputs).
+//
+// piece_cu[k] .. piece_cu[k + 1]: the tokens of piece k (empty behind the last piece);
+// item_first[i]: the first piece of item i.  One thread: a step has a handful of items.
+__global__ void scan_pieces_kernel(const int* __restrict__ cu_tokens, int items, int piece,
+                                   int max_pieces, int* __restrict__ piece_cu,
+                                   int* __restrict__ item_first) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  int at = 0;
+  for (int i = 0; i < items; ++i) {
+    item_first[i] = at;
+    for (int t = cu_tokens[i]; t < cu_tokens[i + 1] && at < max_pieces; t += piece) piece_cu[at++] = t;
+  }
+  item_first[items] = at;
+  for (int k = at; k <= max_pieces; ++k) piece_cu[k] = cu_tokens[items];
+}
+
+// A thread per number of an item's state: S <- the slot's; for the item's pieces in order:
+// E <-> S's place (the piece's start), S <- d^n S + E; the last S goes to the slot.
+__global__ __launch_bounds__(256) void decay_join_kernel(
+    float* __restrict__ piece_states, float* __restrict__ state, const int* __restrict__ piece_cu,
+    const int* __restrict__ item_first, const int* __restrict__ slots,
+    const float* __restrict__ head_decay, int heads, int per_head) {
+  const int item = blockIdx.x, head = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= per_head) return;
+  const int first = item_first[item], last = item_first[item + 1];
+  if (first == last) return;
+  const float d = head_decay[head];
+  float* mine = state + ((int64_t)slots[item] * heads + head) * per_head + e;
+  float s = *mine;
+  for (int k = first; k < last; ++k) {
+    float* record = piece_states + ((int64_t)k * heads + head) * per_head + e;
+    const float left = *record;
+    *record = s;
+    s = fmaf(powf(d, (float)(piece_cu[k + 1] - piece_cu[k])), s, left);
+  }
+  *mine = s;
+}
+
+extern "C" int ps_scan_pieces(const int* cu_tokens, int items, int piece, int max_pieces,
+                              int* piece_cu, int* item_first, void* stream) {
+  PS_REQUIRE(items >= 0 && piece > 0 && max_pieces >= 0, "ps_scan_pieces: bad sizes");
+  hipLaunchKernelGGL(scan_pieces_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, cu_tokens, items,
+                     piece, max_pieces, piece_cu, item_first);
+  PS_CHECK_LAUNCH("ps_scan_pieces");
+  return 0;
+}
+
+extern "C" int ps_decay_join(float* piece_states, float* state, const int* piece_cu,
+                             const int* item_first, const int* slots, const float* head_decay,
+                             int items, int heads, int per_head, void* stream) {
+  PS_REQUIRE(items >= 0 && heads > 0 && per_head > 0, "ps_decay_join: bad sizes");
+  if (items == 0) return 0;
+  hipLaunchKernelGGL(decay_join_kernel, dim3(items, heads, (per_head + 255) / 256), dim3(256), 0,
+                     (hipStream_t)stream, piece_states, state, piece_cu, item_first, slots,
+                     head_decay, heads, per_head);
+  PS_CHECK_LAUNCH("ps_decay_join");
+  return 0;
+}
+
 extern "C" int ps_gla_decay(const float* proj, int64_t ld, int low_col, int rank, const void* w,
                             const float* bias, float tau, float* alpha, int tokens, int channels,
                             int dtype, void* stream) {

@@ -296,6 +296,16 @@ int ps_gla_scan(const float* proj, int64_t ld, int q_col, int k_col, int v_col,
                 const float* alpha, float* state, float* out, const int* cu_tokens,
                 const int* slots, int items, int max_slots, int heads, int key_dim, int value_dim,
                 float q_scale, int longest, const float* head_decay, int silu_inputs, void* stream);
+// Long portions in pieces (recurrences with a decay per head).  ps_scan_pieces cuts the items
+// into pieces of `piece` tokens: piece_cu [max_pieces + 1] (empty pieces behind the last),
+// item_first [items + 1]; max_pieces >= tokens / piece + items.  ps_decay_join: piece_states
+// [max_pieces, heads, per_head] hold what every piece leaves from a zero state and get the
+// state at every piece's start; the slots get the items' last states.
+int ps_scan_pieces(const int* cu_tokens, int items, int piece, int max_pieces, int* piece_cu,
+                   int* item_first, void* stream);
+int ps_decay_join(float* piece_states, float* state, const int* piece_cu, const int* item_first,
+                  const int* slots, const float* head_decay, int items, int heads, int per_head,
+                  void* stream);
 // out[t, :] = rms_norm(o[t, :]) * w * sigmoid(gate[t * gate_ld ...]) over the whole row.
 int ps_row_norm_gate(const float* o, const float* w, float eps, const float* gate, int64_t gate_ld,
                      void* out, int64_t out_stride, int tokens, int columns, int dtype, void* stream);

@@ -46,6 +46,9 @@ _SIGNATURES = {
     "ps_gla_scan": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int,
                     c_void_p],
+    "ps_scan_pieces": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "ps_decay_join": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                      c_void_p],
     "ps_row_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int64, c_int,
                          c_int, c_int, c_void_p],
     "ps_conv_silu": [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -1245,6 +1248,37 @@ def gla_scan(proj, columns, alpha, state, out, cu_tokens, slots, heads, key_dim,
           state.data_ptr(), out.data_ptr(), cu_tokens.data_ptr(), slots.data_ptr(), items,
           state.shape[0], heads, key_dim, value_dim, float(q_scale), int(longest), _ptr(head_decay),
           int(bool(silu_inputs)), _stream())
+
+
+def scan_pieces(cu_tokens, items, piece, max_pieces, piece_cu, item_first):
+    """Cut the step's items into pieces of ``piece`` tokens: ``piece_cu`` (int32, ``max_pieces + 1``:
+    the pieces' token ranges, empty behind the last piece) and ``item_first`` (int32, ``items + 1``).
+    ``max_pieces`` must be at least ``tokens // piece + items``."""
+    _check(cu_tokens, "cu_tokens", torch.int32, 1)
+    _check(piece_cu, "piece_cu", torch.int32, 1)
+    _check(item_first, "item_first", torch.int32, 1)
+    if cu_tokens.numel() != items + 1 or piece_cu.numel() < max_pieces + 1 or item_first.numel() < items + 1:
+        raise KernelError("scan_pieces: an index array is too small")
+    _call("ps_scan_pieces", cu_tokens.data_ptr(), items, int(piece), int(max_pieces), piece_cu.data_ptr(),
+          item_first.data_ptr(), _stream())
+
+
+def decay_join(piece_states, state, piece_cu, item_first, slots, head_decay):
+    """``piece_states`` (float ``[pieces, heads, ...]``): what every piece leaves from a zero state;
+    they get the state at every piece's start, ``state[slot]`` the item's last (``csrc/gla.hip``)."""
+    _check(piece_states, "piece_states", torch.float32)
+    _check(state, "state", torch.float32)
+    heads = state.shape[1]
+    per_head = state[0, 0].numel()
+    if (piece_states.ndim != state.ndim or tuple(piece_states.shape[1:]) != tuple(state.shape[1:])
+            or not (piece_states.is_contiguous() and state.is_contiguous())):
+        raise KernelError("decay_join: the pieces' states must have the slots' shape")
+    _float_vector(head_decay, "head_decay", heads)
+    items = slots.numel()
+    if item_first.numel() < items + 1 or piece_cu.numel() < piece_states.shape[0] + 1:
+        raise KernelError("decay_join: an index array is too small")
+    _call("ps_decay_join", piece_states.data_ptr(), state.data_ptr(), piece_cu.data_ptr(),
+          item_first.data_ptr(), slots.data_ptr(), head_decay.data_ptr(), items, heads, per_head, _stream())
 
 
 def row_norm_gate(o, weight, eps, gate, out):

@@ -131,6 +131,7 @@ class LightningAttention(Mixer):
         self.k_cols = heads * key_dim
         self.v_cols = heads * value_dim
         self._memo_in, self._memo_out = {}, {}
+        self._piece_slots = {}
 
     def parameters(self):
         return {
@@ -152,6 +153,36 @@ class LightningAttention(Mixer):
     def cache_spec(self):
         return SlotStateSpec((self.heads, self.key_dim, self.value_dim), torch.float32)
 
+    # tokens beyond one per item from which a step's items are cut into pieces of PIECE tokens
+    PIECES_FROM = 256
+    PIECE = 128
+
+    def _scan_in_pieces(self, proj, columns, raw, ctx, cache, tokens, items):
+        """The recurrence of a step with long portions: every piece runs the recurrence kernel
+        as an item of its own, first from a zero state (which leaves what the piece adds), then,
+        after the pieces of each item have been joined in order, from its true start for the
+        outputs.  The walk from token to token is as long as a piece, not as a prompt."""
+        workspace = ctx.workspace
+        slots = cache.state.shape[0]
+        most = workspace.max_rows // self.PIECE + slots          # no step has more pieces
+        pieces = tokens // self.PIECE + items
+        piece_cu = workspace.flat("lightning_piece_cu", most + 1, torch.int32)
+        item_first = workspace.flat("lightning_item_first", slots + 1, torch.int32)
+        states = workspace.flat("lightning_piece_states", most * cache.state[0].numel(), torch.float32)
+        states = states[:pieces * cache.state[0].numel()].view((pieces,) + tuple(cache.state.shape[1:]))
+        own_slots = self._piece_slots.get((workspace.serial, pieces))
+        if own_slots is None:
+            own_slots = self._piece_slots[(workspace.serial, pieces)] = torch.arange(
+                pieces, dtype=torch.int32, device=proj.device)
+        kernels.scan_pieces(ctx.cu_tokens, items, self.PIECE, pieces, piece_cu, item_first)
+        piece_cu = piece_cu[:pieces + 1]
+        states.zero_()
+        for turn in range(2):
+            kernels.gla_scan(proj, columns, None, states, raw, piece_cu, own_slots, self.heads,
+                             self.key_dim, self.value_dim, 1.0, head_decay=self.head_decay)
+            if turn == 0:
+                kernels.decay_join(states, cache.state, piece_cu, item_first, ctx.slots, self.head_decay)
+
     def forward(self, x, residual, ctx, cache):
         tokens = ctx.tokens
         k_col, v_col = self.k_cols, 2 * self.k_cols
@@ -165,10 +196,14 @@ class LightningAttention(Mixer):
         # recurrence waits for every piece that it stages, a launch ahead of it is faster
         if not ctx.decode_only:
             kernels.silu_columns(proj, 0, gate_col)
-        kernels.gla_scan(proj, (0, k_col, v_col), None, cache.state, raw, ctx.cu_tokens, ctx.slots,
-                         self.heads, self.key_dim, self.value_dim, 1.0,
-                         longest=1 if ctx.decode_only else 0, head_decay=self.head_decay,
-                         silu_inputs=ctx.decode_only)
+        items = ctx.slots.numel()
+        if tokens - items >= self.PIECES_FROM:
+            self._scan_in_pieces(proj, (0, k_col, v_col), raw, ctx, cache, tokens, items)
+        else:
+            kernels.gla_scan(proj, (0, k_col, v_col), None, cache.state, raw, ctx.cu_tokens, ctx.slots,
+                             self.heads, self.key_dim, self.value_dim, 1.0,
+                             longest=1 if ctx.decode_only else 0, head_decay=self.head_decay,
+                             silu_inputs=ctx.decode_only)
         gated = workspace.first_rows("lightning_out", self.v_cols, self.dtype, tokens)
         kernels.row_norm_gate(raw, self.norm_gamma, self.norm_eps,
                               proj[:, gate_col:gate_col + self.v_cols], gated)

@@ -335,6 +335,44 @@ def test_recurrence_with_a_decay_per_head_and_activated_inputs(heads, dim, vdim)
     assert torch.allclose(state[0].double().cpu(), finals[0], atol=1e-3, rtol=2e-4)
 
 
+@pytest.mark.parametrize("heads,dim,vdim", [(2, 16, 24), (3, 64, 64)])
+def test_recurrence_with_a_decay_per_head_in_pieces_side_by_side(heads, dim, vdim):
+    """The mixer's way with long portions (every piece of 128 tokens an item of its own, joined in
+    order) against the walk of one block per item: items of unequal length, one shorter than a
+    piece, one of a whole number of pieces, from states that are not zero."""
+    import types
+
+    from pagedserve_amd.parts import Workspace
+    from pagedserve_amd.parts.linear_attention import LightningAttention
+
+    kernels = _kernels()
+    g = torch.Generator().manual_seed(dim)
+    lengths, slots = [300, 40, 256, 1], [3, 0, 1, 4]
+    total = sum(lengths)
+    k_col, v_col = heads * dim, 2 * heads * dim
+    proj = (torch.randn((total, v_col + heads * vdim), generator=g) * 0.5).cuda()
+    decay = [0.999, 0.9, 0.97][:heads]
+    mixer = LightningAttention(64, torch.float32, heads, dim, vdim, decay, 1e-5)
+    mixer.head_decay = torch.tensor(decay, device="cuda")
+    start = torch.randn((5, heads, dim, vdim), generator=g).cuda()
+    cu = [0]
+    for length in lengths:
+        cu.append(cu[-1] + length)
+    whole_state, whole_out = start.clone(), torch.empty((total, heads * vdim), device="cuda")
+    kernels.gla_scan(proj, (0, k_col, v_col), None, whole_state, whole_out, _ints(cu), _ints(slots), heads, dim,
+                     vdim, 1.0, head_decay=mixer.head_decay)
+    ctx = types.SimpleNamespace(workspace=Workspace(total + 50, "cuda"), cu_tokens=_ints(cu), slots=_ints(slots))
+    cache = types.SimpleNamespace(state=start.clone())
+    out = torch.full((total, heads * vdim), float("nan"), device="cuda")
+    for _ in range(2):      # (the second time the scratch holds what the first left)
+        cache.state.copy_(start)
+        mixer._scan_in_pieces(proj, (0, k_col, v_col), out, ctx, cache, total, len(lengths))
+        scale = float(whole_out.abs().max())
+        assert float((out - whole_out).abs().max()) <= 2e-5 * scale
+        assert torch.allclose(cache.state, whole_state, atol=1e-3, rtol=2e-4)
+    assert torch.equal(cache.state[2], start[2])      # a slot that no item holds
+
+
 def test_norm_over_all_heads_with_a_sigmoid_gate():
     kernels = _kernels()
     g = torch.Generator().manual_seed(9)
@@ -468,6 +506,24 @@ def test_a_loud_key_just_inside_and_just_outside_the_window(tmp_path, window, dt
         rows = helpers.replay_in_process(engine, steps)
         worst, scale, where = helpers.max_error(rows, reference)
         assert worst <= TOLERANCE[dtype] * scale, (name, worst / scale, where)
+        engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "C"])
+def test_long_portions_whose_recurrences_run_in_pieces(tmp_path, which, dtype):
+    """Prompts of several hundred tokens whole and in long portions beside a short one: the
+    recurrent mixers cut such steps into pieces that run side by side."""
+    folder, raw, tensors, page_size = zetunex_models.folder_of(tmp_path, which)
+    requests = _requests(raw, (520, 300, 9), 23)
+    reference = _reference(raw, tensors, requests)
+    for name, steps in (("whole", helpers.trace_whole(requests)),
+                        ("portions", helpers.trace_portions(requests, sizes=(260, 2, 131, 300))),
+                        ("mixed", helpers.trace_mixed(requests, max_live=3, portion=(270, 129), decode_tail=3))):
+        engine = _engine(folder, dtype, page_size, steps, max_requests=3)
+        rows = helpers.replay_in_process(engine, steps)
+        good, what = _close(rows, reference, dtype)
+        assert good, (which, name, what)
         engine.cache.check_invariants()
 
 
