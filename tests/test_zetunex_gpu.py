@@ -527,6 +527,24 @@ def test_long_portions_whose_recurrences_run_in_pieces(tmp_path, which, dtype):
         engine.cache.check_invariants()
 
 
+def test_a_recorded_step_of_a_long_portion_replays_right(tmp_path):
+    """A step of one long prompt is recorded as a graph once its layout keeps coming back; every
+    replay (pieces, joins, sorted experts and cleared scratch inside it) gives what the plain
+    implementation gives for that request's own tokens."""
+    folder, raw, tensors, page_size = zetunex_models.folder_of(tmp_path, "A")
+    requests = _requests(raw, (300,) * 7, 61)
+    reference = _reference(raw, tensors, requests)
+    steps = helpers.trace_whole(requests)
+    engine = _engine(folder, "float32", page_size, steps, max_requests=2)
+    engine.record_after = 2
+    rows = helpers.replay_in_process(engine, steps)
+    assert engine.graph_summary()["graph_replays"] >= 3
+    for rid in requests:
+        mine = {key: row for key, row in rows.items() if key[0] == rid}
+        worst, scale, where = helpers.max_error(mine, reference)
+        assert worst <= TOLERANCE["float32"] * scale, (rid, worst / scale, where)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_over_many_pages_and_graph_replays(tmp_path, dtype):
     folder, raw, tensors, _ = zetunex_models.folder_of(tmp_path, "A")
