@@ -40,7 +40,7 @@ def test_stream_step_adds_norms_and_clears(width):
     y = torch.randn((tokens, width), generator=g, dtype=F64)
     bias = torch.randn(width, generator=g, dtype=F64)
     gamma = 1 + 0.2 * torch.randn(width, generator=g, dtype=F64)
-    eps, factor = 1e-5, 0.3
+    eps, factor = 1e-5, 0.35
     for dtype in (torch.float32, torch.bfloat16):
         dh, dy = _gpu(h), _gpu(y)
         normed = torch.full((tokens, width), float("nan"), dtype=dtype, device="cuda")
@@ -83,7 +83,7 @@ def test_gate_product_and_pair_of_norms():
     assert float(da.abs().max()) == 0.0 and float(db.abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("experts,groups,keep,top", [(8, 4, 2, 3), (16, 2, 1, 3), (6, 1, 1, 6), (12, 6, 3, 1),
+@pytest.mark.parametrize("experts,groups,keep,top", [(8, 4, 2, 3), (18, 3, 1, 4), (6, 1, 1, 6), (12, 6, 3, 1),
                                                      (5, 5, 2, 2), (64, 8, 4, 8), (128, 8, 4, 6), (66, 3, 2, 30)])
 def test_router_chooses_within_the_best_groups(experts, groups, keep, top):
     kernels = _kernels()
@@ -93,10 +93,10 @@ def test_router_chooses_within_the_best_groups(experts, groups, keep, top):
     router = torch.randn((experts, width), generator=g) * 0.5
     # one row whose best expert sits in a group that is otherwise poor, next to a group of good ones
     logits = x.double() @ router.double().T
-    chosen, weights = plain.route(logits, groups, keep, top, 2.5)
+    chosen, weights = plain.route(logits, groups, keep, top, 1.75)
     ids = torch.full((tokens, top), -1, dtype=torch.int32, device="cuda")
     got = torch.zeros((tokens, top), device="cuda")
-    kernels.moe_route(x.cuda(), router.cuda(), groups, keep, top, 2.5, ids, got)
+    kernels.moe_route(x.cuda(), router.cuda(), groups, keep, top, 1.75, ids, got)
     ids, got = ids.cpu(), got.double().cpu()
     for t in range(tokens):
         assert sorted(ids[t].tolist()) == sorted(chosen[t]), t
